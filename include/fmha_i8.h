@@ -1,0 +1,83 @@
+/*
+ * C ABI of the MI355X (gfx950) INT8 fused multi-head flash-attention launch path.
+ *
+ * The library (libfmha_i8.so) exports plain C symbols: pointers, PODs by value and a HIP stream handle.  No C++
+ * types, no torch types.  A C++ caller that was written against the reference's `gpuImpl::FMHAInferI8`
+ * (inc/fmha_i8.h:7-15) compiles unchanged against the forwarding wrapper at the bottom of this header; the only
+ * difference is that the stream is a hipStream_t.
+ *
+ * Data contract (reference: src/fmha_i8.cu:157-173, inc/fmha_i8.cuh:45,88-89,112-114,325):
+ *   q, k, v, o     int8, device memory, [batch_num, head_num, seq_len, head_dim] row-major contiguous,
+ *                  base pointers 16-byte aligned (hipMalloc gives 256); o must not alias an input.
+ *   padding_mask   int8, device memory, [batch_num, seq_len] over key positions; a NONZERO byte means the key is
+ *                  masked OUT (inc/fmha_i8.cuh:189-192).  No alignment requirement.
+ *   ownership      caller owns every buffer; the callee allocates nothing, frees nothing, keeps no pointer.
+ *   asynchrony     one kernel is enqueued on `stream`; the call returns immediately and never synchronises.
+ *   threading      no mutable global state: callable concurrently from any host thread.
+ *
+ * Supported shapes: head_dim in {64, 128}; seq_len a positive multiple of 128; batch_num, head_num >= 1.
+ * (The reference's ladder, src/fmha_i8.cu:39-154, covers head_dim in {64,128} and eleven fixed seq_len values;
+ * every one of its 128-multiples is covered here, and so is any other multiple of 128.)
+ *
+ * Numerics follow the reference kernel (inc/fmha_i8.cuh:71-72,181-253,298-332): int32 Q.K^T, 1/sqrt(d) and
+ * q_amax*k_amax/127^2 dequantisation, softmax over blocks of 128 keys with the BLOCK-LOCAL row maximum,
+ * P requantised to int8 in [-128, 0] with scale -128, int32 P.V, online (m, l, O) merge, O requantised with
+ * v_amax/(128*o_amax), round-half-even, clamp to [-127, 127].  Rows whose keys are all masked produce 0.
+ */
+#ifndef FMHA_I8_H_
+#define FMHA_I8_H_
+
+#include <hip/hip_runtime_api.h>
+#include "fmha_param_i8.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes of FMHAInferI8Status.  Values >= 1000 are 1000 + the hipError_t of the failed launch. */
+#define FMHA_I8_OK 0
+#define FMHA_I8_ERR_NULL_POINTER 1   /* q, k, v, padding_mask or o is NULL */
+#define FMHA_I8_ERR_HEAD_DIM 2       /* head_dim not in {64, 128} */
+#define FMHA_I8_ERR_SEQ_LEN 3        /* seq_len <= 0 or not a multiple of 128 */
+#define FMHA_I8_ERR_BATCH_HEAD 4     /* batch_num or head_num <= 0, or the grid would exceed HIP limits */
+#define FMHA_I8_ERR_ALIGNMENT 5      /* q, k, v or o not 16-byte aligned */
+#define FMHA_I8_ERR_SCALE 6          /* an amax is not finite, or o_amax <= 0 */
+#define FMHA_I8_ERR_HIP_BASE 1000
+
+/* Replaces gpuImpl::FMHAInferI8 (inc/fmha_i8.h:7-15, src/fmha_i8.cu:157-173).
+ * Same argument list and meaning; returns nothing, like the reference.  On an unsupported shape the reference
+ * silently launches nothing (src/fmha_i8.cu:39-154); this entry point also leaves `o` untouched, and additionally
+ * writes one diagnostic line to stderr.  `use_tcu` is accepted for signature compatibility: the reference's
+ * `false` path is an empty kernel (inc/fmha_i8.cuh:337-342); here both values run the MFMA kernel. */
+void FMHAInferI8(hipStream_t stream, FMHAParamI8 fmha_param, AttnDataDescriptor attn_desc, const void* q,
+                 const void* k, const void* v, const void* padding_mask, void* o, bool use_tcu);
+
+/* Same operation, but reports what the reference cannot (its launch is unchecked, src/fmha_i8.cu:82-84):
+ * FMHA_I8_OK, one of FMHA_I8_ERR_*, or FMHA_I8_ERR_HIP_BASE + hipError_t.  Never prints, never aborts. */
+int FMHAInferI8Status(hipStream_t stream, FMHAParamI8 fmha_param, AttnDataDescriptor attn_desc, const void* q,
+                      const void* k, const void* v, const void* padding_mask, void* o, bool use_tcu);
+
+/* Argument check only (no HIP call at all): what FMHAInferI8Status would return before launching.
+ * Stands in for the reference's if/else ladder over (head_dim, seq_len) (src/fmha_i8.cu:39-154). */
+int FMHAInferI8CheckArgs(FMHAParamI8 fmha_param, AttnDataDescriptor attn_desc, const void* q, const void* k,
+                         const void* v, const void* padding_mask, const void* o);
+
+/* Human-readable text for a status code returned by the two functions above (static storage). */
+const char* FMHAInferI8StatusString(int status);
+
+/* Library build identification: "fmha_i8 gfx950 <variant>" (static storage). */
+const char* FMHAInferI8Version(void);
+
+#ifdef __cplusplus
+} /* extern "C" */
+
+/* Source compatibility with call sites written for the reference (test_fmha_i8.cpp:204,207,219,222). */
+namespace gpuImpl {
+inline void FMHAInferI8(hipStream_t stream, FMHAParamI8 fmha_param, AttnDataDescriptor attn_desc, const void* q,
+                        const void* k, const void* v, const void* padding_mask, void* o, const bool use_tcu) {
+  ::FMHAInferI8(stream, fmha_param, attn_desc, q, k, v, padding_mask, o, use_tcu);
+}
+}  // namespace gpuImpl
+#endif
+
+#endif /* FMHA_I8_H_ */

@@ -1,0 +1,146 @@
+"""Host-side mirror (Python) of the INT8 fused attention launch API on MI355X.
+
+The product is the C-ABI library ``libfmha_i8.so`` built from ``csrc/`` (see ``include/fmha_i8.h``).  This module binds
+it with ctypes and keeps the reference's names and argument order (inc/fmha_i8.h:7-15, inc/fmha_param_i8.h:3-17):
+
+    FMHAInferI8(stream, fmha_param, attn_desc, q, k, v, padding_mask, o, use_tcu)
+
+``q, k, v, padding_mask, o`` are device pointers (ints) or objects with ``data_ptr()`` (torch tensors on the GPU);
+``stream`` is a ``hipStream_t`` value (int), a ``torch.cuda.Stream`` or None for the null stream.  There is no CPU
+fallback: if the library is missing or cannot be loaded, every call raises.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libfmha_i8.so")
+
+EXPORTED_SYMBOLS = ("FMHAInferI8", "FMHAInferI8Status", "FMHAInferI8CheckArgs", "FMHAInferI8StatusString",
+                    "FMHAInferI8Version")
+
+FMHA_I8_OK = 0
+FMHA_I8_ERR_NULL_POINTER = 1
+FMHA_I8_ERR_HEAD_DIM = 2
+FMHA_I8_ERR_SEQ_LEN = 3
+FMHA_I8_ERR_BATCH_HEAD = 4
+FMHA_I8_ERR_ALIGNMENT = 5
+FMHA_I8_ERR_SCALE = 6
+FMHA_I8_ERR_HIP_BASE = 1000
+
+
+class AttnDataDescriptor(C.Structure):
+    """inc/fmha_param_i8.h:3-8 — same field order and defaults."""
+    _fields_ = [("batch_num", C.c_int), ("seq_len", C.c_int), ("head_num", C.c_int), ("head_dim", C.c_int)]
+
+    def __init__(self, batch_num=1, seq_len=64, head_num=4, head_dim=64):
+        super().__init__(batch_num, seq_len, head_num, head_dim)
+
+
+class FMHAParamI8(C.Structure):
+    """inc/fmha_param_i8.h:10-17 — same field order and defaults; s_max is carried but unused."""
+    _fields_ = [("q_amax", C.c_float), ("k_amax", C.c_float), ("v_amax", C.c_float), ("o_amax", C.c_float),
+                ("s_max", C.c_float)]
+
+    def __init__(self, q_amax=0.0, k_amax=0.0, v_amax=0.0, o_amax=1.0, s_max=1.0):
+        super().__init__(q_amax, k_amax, v_amax, o_amax, s_max)
+
+
+class FMHAError(RuntimeError):
+    def __init__(self, status, text):
+        super().__init__("FMHAInferI8 failed with status %d: %s" % (status, text))
+        self.status = status
+
+
+_lib = None
+
+
+def load_library(path=None):
+    """dlopen libfmha_i8.so and declare the prototypes of include/fmha_i8.h.  Raises if the library is absent."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    p = path or LIB_PATH
+    if not os.path.exists(p):
+        raise FileNotFoundError(
+            "%s is not built; run `python -c 'import __graft_entry__ as g; g.build()'` at the repository root "
+            "(there is no CPU fallback for this path)" % p)
+    L = C.CDLL(p)
+    ptr = C.c_void_p
+    L.FMHAInferI8.argtypes = [ptr, FMHAParamI8, AttnDataDescriptor, ptr, ptr, ptr, ptr, ptr, C.c_bool]
+    L.FMHAInferI8.restype = None
+    L.FMHAInferI8Status.argtypes = L.FMHAInferI8.argtypes
+    L.FMHAInferI8Status.restype = C.c_int
+    L.FMHAInferI8CheckArgs.argtypes = [FMHAParamI8, AttnDataDescriptor, ptr, ptr, ptr, ptr, ptr]
+    L.FMHAInferI8CheckArgs.restype = C.c_int
+    L.FMHAInferI8StatusString.argtypes = [C.c_int]
+    L.FMHAInferI8StatusString.restype = C.c_char_p
+    L.FMHAInferI8Version.argtypes = []
+    L.FMHAInferI8Version.restype = C.c_char_p
+    if path is None:
+        _lib = L
+    return L
+
+
+def _ptr(x):
+    if x is None:
+        return None
+    if hasattr(x, "data_ptr"):
+        return x.data_ptr()
+    return int(x)
+
+
+def _stream(s):
+    if s is None:
+        return None
+    if hasattr(s, "cuda_stream"):
+        return s.cuda_stream
+    return int(s)
+
+
+def FMHAInferI8(stream, fmha_param, attn_desc, q, k, v, padding_mask, o, use_tcu=True):
+    """Drop-in for gpuImpl::FMHAInferI8 (src/fmha_i8.cu:157-173): enqueue, return nothing, never synchronise."""
+    load_library().FMHAInferI8(_stream(stream), fmha_param, attn_desc, _ptr(q), _ptr(k), _ptr(v), _ptr(padding_mask),
+                               _ptr(o), bool(use_tcu))
+
+
+def FMHAInferI8Status(stream, fmha_param, attn_desc, q, k, v, padding_mask, o, use_tcu=True):
+    """Same launch, returning the status code of include/fmha_i8.h."""
+    return int(load_library().FMHAInferI8Status(_stream(stream), fmha_param, attn_desc, _ptr(q), _ptr(k), _ptr(v),
+                                                _ptr(padding_mask), _ptr(o), bool(use_tcu)))
+
+
+def FMHAInferI8CheckArgs(fmha_param, attn_desc, q, k, v, padding_mask, o):
+    return int(load_library().FMHAInferI8CheckArgs(fmha_param, attn_desc, _ptr(q), _ptr(k), _ptr(v),
+                                                   _ptr(padding_mask), _ptr(o)))
+
+
+def status_string(status):
+    return load_library().FMHAInferI8StatusString(int(status)).decode()
+
+
+def version():
+    return load_library().FMHAInferI8Version().decode()
+
+
+def fmha_infer_i8(q, k, v, padding_mask, q_amax, k_amax, v_amax, o_amax=1.0, out=None, stream=None):
+    """Convenience over FMHAInferI8Status for torch int8 tensors on the GPU.
+
+    q, k, v: int8 [B, H, S, d] contiguous; padding_mask: int8 [B, S], nonzero = key masked out
+    (inc/fmha_i8.cuh:189-192).  Returns int8 O [B, H, S, d].  Raises FMHAError on a nonzero status."""
+    import torch
+
+    for name, t in (("q", q), ("k", k), ("v", v), ("padding_mask", padding_mask)):
+        if not (t.is_cuda and t.dtype == torch.int8 and t.is_contiguous()):
+            raise ValueError("%s must be a contiguous int8 tensor on the GPU" % name)
+    B, H, S, d = q.shape
+    if k.shape != q.shape or v.shape != q.shape or tuple(padding_mask.shape) != (B, S):
+        raise ValueError("shape mismatch: q/k/v [B,H,S,d] and padding_mask [B,S] expected")
+    if out is None:
+        out = torch.empty_like(q)
+    if stream is None:
+        stream = torch.cuda.current_stream(q.device)
+    st = FMHAInferI8Status(stream, FMHAParamI8(q_amax, k_amax, v_amax, o_amax, 1.0), AttnDataDescriptor(B, S, H, d),
+                           q, k, v, padding_mask, out, True)
+    if st != FMHA_I8_OK:
+        raise FMHAError(st, status_string(st))
+    return out

@@ -1,0 +1,102 @@
+// C ABI of libfmha_i8.so: argument checking, scale folding and the kernel launch.  Stands where the reference has
+// FMHAInferI8 / LaunchFMHAInfer_TCU (src/fmha_i8.cu:31-173): the if/else ladder over (head_dim, seq_len) template
+// instantiations becomes a run-time seq_len and a two-way switch on head_dim.
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/fmha_i8.h"
+#include "fmha_i8_kernel.hip"
+
+namespace {
+
+using fmha_i8_gfx950::KernelArgs;
+
+int check_args(const FMHAParamI8& p, const AttnDataDescriptor& a, const void* q, const void* k, const void* v,
+               const void* mask, const void* o) {
+  if (!q || !k || !v || !mask || !o) return FMHA_I8_ERR_NULL_POINTER;
+  if (a.head_dim != 64 && a.head_dim != 128) return FMHA_I8_ERR_HEAD_DIM;
+  if (a.seq_len <= 0 || a.seq_len % fmha_i8_gfx950::kBlockK != 0) return FMHA_I8_ERR_SEQ_LEN;
+  if (a.batch_num <= 0 || a.head_num <= 0) return FMHA_I8_ERR_BATCH_HEAD;
+  const long long wgs = (long long)a.batch_num * a.head_num * (a.seq_len / fmha_i8_gfx950::kBlockQ);
+  if (wgs > 0x7fffffffLL) return FMHA_I8_ERR_BATCH_HEAD;
+  const uintptr_t bits = (uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o;
+  if (bits & 15u) return FMHA_I8_ERR_ALIGNMENT;
+  if (!isfinite(p.q_amax) || !isfinite(p.k_amax) || !isfinite(p.v_amax) || !isfinite(p.o_amax) || !(p.o_amax > 0.f))
+    return FMHA_I8_ERR_SCALE;
+  return FMHA_I8_OK;
+}
+
+int launch(hipStream_t stream, const FMHAParamI8& p, const AttnDataDescriptor& a, const void* q, const void* k,
+           const void* v, const void* mask, void* o) {
+  const int st = check_args(p, a, q, k, v, mask, o);
+  if (st != FMHA_I8_OK) return st;
+  constexpr float kLog2e = 1.4426950408889634f;
+  KernelArgs args;
+  args.q = static_cast<const int8_t*>(q);
+  args.k = static_cast<const int8_t*>(k);
+  args.v = static_cast<const int8_t*>(v);
+  args.mask = static_cast<const int8_t*>(mask);
+  args.o = static_cast<int8_t*>(o);
+  args.seq_len = a.seq_len;
+  args.head_num = a.head_num;
+  args.q_blocks = a.seq_len / fmha_i8_gfx950::kBlockQ;
+  args.total_wgs = a.batch_num * a.head_num * args.q_blocks;
+  // inc/fmha_i8.cuh:71-72: row_scale = 1/sqrt(d), scale_qk_out = q_amax*k_amax/127^2; folded with log2(e).
+  const float row_scale = 1.0f / sqrtf((float)a.head_dim);
+  const float scale_qk_out = p.q_amax * p.k_amax / (127.f * 127.f);
+  args.c2 = row_scale * scale_qk_out * kLog2e;
+  args.floor2 = -1e6f * kLog2e;
+  args.masked2 = -1000000.f * args.c2;
+  args.out_scale = p.v_amax / (p.o_amax * 128.f);  // inc/fmha_i8.cuh:318
+  const dim3 grid((unsigned)args.total_wgs), block(fmha_i8_gfx950::kThreads);
+  if (a.head_dim == 128)
+    hipLaunchKernelGGL(fmha_i8_gfx950::fmha_i8_fwd_kernel<128>, grid, block, 0, stream, args);
+  else
+    hipLaunchKernelGGL(fmha_i8_gfx950::fmha_i8_fwd_kernel<64>, grid, block, 0, stream, args);
+  const hipError_t err = hipGetLastError();
+  return err == hipSuccess ? FMHA_I8_OK : FMHA_I8_ERR_HIP_BASE + (int)err;
+}
+
+}  // namespace
+
+extern "C" {
+
+int FMHAInferI8CheckArgs(FMHAParamI8 fmha_param, AttnDataDescriptor attn_desc, const void* q, const void* k,
+                         const void* v, const void* padding_mask, const void* o) {
+  return check_args(fmha_param, attn_desc, q, k, v, padding_mask, o);
+}
+
+int FMHAInferI8Status(hipStream_t stream, FMHAParamI8 fmha_param, AttnDataDescriptor attn_desc, const void* q,
+                      const void* k, const void* v, const void* padding_mask, void* o, bool /*use_tcu*/) {
+  return launch(stream, fmha_param, attn_desc, q, k, v, padding_mask, o);
+}
+
+void FMHAInferI8(hipStream_t stream, FMHAParamI8 fmha_param, AttnDataDescriptor attn_desc, const void* q, const void* k,
+                 const void* v, const void* padding_mask, void* o, bool /*use_tcu*/) {
+  const int st = launch(stream, fmha_param, attn_desc, q, k, v, padding_mask, o);
+  if (st != FMHA_I8_OK)
+    fprintf(stderr, "FMHAInferI8: nothing launched, o left untouched: %s (B=%d H=%d S=%d d=%d)\n",
+            FMHAInferI8StatusString(st), attn_desc.batch_num, attn_desc.head_num, attn_desc.seq_len,
+            attn_desc.head_dim);
+}
+
+const char* FMHAInferI8StatusString(int status) {
+  switch (status) {
+    case FMHA_I8_OK: return "ok";
+    case FMHA_I8_ERR_NULL_POINTER: return "null pointer argument";
+    case FMHA_I8_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
+    case FMHA_I8_ERR_SEQ_LEN: return "seq_len must be a positive multiple of 128";
+    case FMHA_I8_ERR_BATCH_HEAD: return "batch_num and head_num must be positive (and the grid must fit)";
+    case FMHA_I8_ERR_ALIGNMENT: return "q, k, v and o must be 16-byte aligned";
+    case FMHA_I8_ERR_SCALE: return "amax values must be finite and o_amax > 0";
+    default: break;
+  }
+  if (status >= FMHA_I8_ERR_HIP_BASE) return hipGetErrorString((hipError_t)(status - FMHA_I8_ERR_HIP_BASE));
+  return "unknown status";
+}
+
+const char* FMHAInferI8Version(void) { return "fmha_i8 gfx950 mfma32x32x32-lds-swizzle"; }
+
+}  // extern "C"
