@@ -64,6 +64,13 @@ def load_library(path=None):
         raise FileNotFoundError(
             "%s is not built; run `python -c 'import __graft_entry__ as g; g.build()'` at the repository root "
             "(there is no CPU fallback for this path)" % p)
+    # A process must hold ONE HIP runtime.  PyTorch-ROCm wheels carry their own libamdhip64.so.7; importing torch first
+    # makes the dynamic linker satisfy this library's libamdhip64.so.7 dependency with that already-loaded copy.  The
+    # opposite order (system runtime first, torch's second) leaves the process with a runtime that finds no device.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     L = C.CDLL(p)
     ptr = C.c_void_p
     L.FMHAInferI8.argtypes = [ptr, FMHAParamI8, AttnDataDescriptor, ptr, ptr, ptr, ptr, ptr, C.c_bool]

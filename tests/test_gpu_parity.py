@@ -1,0 +1,262 @@
+"""GPU parity tests proper: the HIP kernel, called through the C ABI of libfmha_i8.so, against the CPU checker on the
+same seeded inputs.  Gate (int8 O): within +-1 LSB on >= 99.9 % of elements and max |delta| <= 2."""
+import glob
+import os
+
+import numpy as np
+import pytest
+
+import fmha_cases as fc
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+WITHIN1_MIN = 0.999  # tolerance of the gate, in fractions of elements within +-1 LSB
+MAX_ABS_LSB = 2
+
+
+def to_dev(dev, *arrays):
+    import torch
+    return [torch.from_numpy(np.ascontiguousarray(a)).to(dev) for a in arrays]
+
+
+def gpu_run(pkg, dev, c, **scales):
+    import torch
+    s = dict(q_amax=c["q_amax"], k_amax=c["k_amax"], v_amax=c["v_amax"], o_amax=c["o_amax"])
+    s.update(scales)
+    q, k, v, m = to_dev(dev, c["q"], c["k"], c["v"], c["mask"])
+    o = pkg.fmha_infer_i8(q, k, v, m, s["q_amax"], s["k_amax"], s["v_amax"], s["o_amax"])
+    torch.cuda.synchronize()
+    return o.cpu().numpy()
+
+
+def cpu_run(orc, c, heads=None, **scales):
+    s = dict(q_amax=c["q_amax"], k_amax=c["k_amax"], v_amax=c["v_amax"], o_amax=c["o_amax"])
+    s.update(scales)
+    return orc.fmha_i8_blockwise(c["q"], c["k"], c["v"], c["mask"], s["q_amax"], s["k_amax"], s["v_amax"], s["o_amax"],
+                                 heads=heads)
+
+
+def check(got, want, what):
+    st = fc.parity_stats(got, want)
+    print(what, st, flush=True)
+    assert st["within1"] >= WITHIN1_MIN and st["max"] <= MAX_ABS_LSB, (what, st)
+    return st
+
+
+# ---- committed known-answer fixtures -----------------------------------------------------------------------------
+FIXTURES = sorted(glob.glob(os.path.join(HERE, "golden", "*.npz")))
+
+
+@pytest.mark.parametrize("path", FIXTURES, ids=[os.path.basename(p) for p in FIXTURES])
+def test_golden_fixture(pkg, dev, path):
+    f = np.load(path)
+    qa, ka, va, oa = (float(x) for x in f["amax"])
+    c = dict(q=f["q"], k=f["k"], v=f["v"], mask=f["mask"], q_amax=qa, k_amax=ka, v_amax=va, o_amax=oa)
+    check(gpu_run(pkg, dev, c), f["o"], os.path.basename(path))
+
+
+# ---- the reference's own sweep (test_fmha_i8.cpp:295-309: B=H=1, d in {64,128}) on the 128-multiples, reference-style
+# data (uniform +-0.5, V = |u|, scattered 20 % mask, o_amax measured from the float path), both criteria ---------------
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("S", [128, 256, 384, 512, 1024])
+def test_reference_sweep(pkg, orc, dev, S, d):
+    c = fc.make_inputs(1, 1, S, d, dist="reference", pad="scatter", seed=31)
+    o_ref = orc.fmha_fp32(c["qf"], c["kf"], c["vf"], c["mask"])
+    c["o_amax"] = orc.abs_max(o_ref)  # test_fmha_i8.cpp:161
+    got = gpu_run(pkg, dev, c)
+    check(got, cpu_run(orc, c), "sweep S=%d d=%d" % (S, d))
+    dev_pct = orc.mean_rel_deviation_pct(got, o_ref, c["o_amax"])
+    assert dev_pct < 20.0, dev_pct  # inc/utils.hpp:88
+
+
+# ---- the five benchmark configurations -----------------------------------------------------------------------------
+def test_config_c1_all_heads(pkg, orc, dev):
+    c = fc.make_config("C1")
+    check(gpu_run(pkg, dev, c), cpu_run(orc, c), "C1")
+
+
+def test_config_c2_all_heads(pkg, orc, dev):
+    c = fc.make_config("C2")
+    assert c["mask"].any()
+    check(gpu_run(pkg, dev, c), cpu_run(orc, c), "C2")
+
+
+@pytest.mark.parametrize("name,heads", [("C3", (0, 64)), ("C4", (5, 9)), ("C5", (250, 256))])
+def test_large_configs_on_sampled_heads(pkg, orc, dev, name, heads):
+    # full-size run on the GPU; the checker finishes a head range in seconds
+    c = fc.make_config(name)
+    got = gpu_run(pkg, dev, c)
+    want = cpu_run(orc, c, heads=heads)
+    B, H, S, d = c["q"].shape
+    sl = slice(heads[0], heads[1])
+    check(got.reshape(B * H, S, d)[sl], want.reshape(B * H, S, d)[sl], name)
+
+
+# ---- size-independent properties at full benchmark size (no CPU pass needed) ----------------------------------------
+def test_full_size_properties_c3(pkg, dev):
+    import torch
+    c = fc.make_config("C3")
+    base = gpu_run(pkg, dev, c)
+    # determinism: same call, same bits
+    assert np.array_equal(gpu_run(pkg, dev, c), base)
+    # head/batch independence: a [1,1] call on one head equals that head of the full call, bit for bit
+    for b, h in ((0, 0), (3, 15), (2, 7)):
+        one = dict(c, q=c["q"][b:b + 1, h:h + 1], k=c["k"][b:b + 1, h:h + 1], v=c["v"][b:b + 1, h:h + 1],
+                   mask=c["mask"][b:b + 1])
+        assert np.array_equal(gpu_run(pkg, dev, one)[0, 0], base[b, h])
+    # only q_amax*k_amax and v_amax/o_amax matter
+    alt = gpu_run(pkg, dev, c, q_amax=c["q_amax"] * 2, k_amax=c["k_amax"] / 2, v_amax=c["v_amax"] * 4, o_amax=4.0)
+    assert np.array_equal(alt, base)
+    # permuting the key blocks (K and V together) changes only float merge order
+    S = c["q"].shape[2]
+    order = np.random.default_rng(5).permutation(S // 128)
+    idx = np.concatenate([np.arange(128) + 128 * b for b in order])
+    perm = dict(c, k=np.ascontiguousarray(c["k"][:, :, idx]), v=np.ascontiguousarray(c["v"][:, :, idx]))
+    st = fc.parity_stats(gpu_run(pkg, dev, perm), base)
+    assert st["within1"] >= 0.9999 and st["max"] <= 1, st
+    # Q == 0: uniform attention, closed form rne(clamp(v_amax/o_amax * mean V))
+    z = dict(c, q=np.zeros_like(c["q"]))
+    got = gpu_run(pkg, dev, z, v_amax=2.0, o_amax=1.0).astype(np.int64)
+    y = 2.0 * c["v"].astype(np.float64).mean(axis=2, keepdims=True)
+    want = np.broadcast_to(np.clip(np.rint(y), -127, 127), got.shape)
+    assert np.abs(got - want).max() <= 1 and (got == want).mean() > 0.99
+    del torch
+
+
+def test_full_size_mask_properties_c4(pkg, dev):
+    c = fc.make_config("C4")
+    base = gpu_run(pkg, dev, c)
+    # keys behind the mask cannot change a bit
+    rng = np.random.default_rng(6)
+    c2 = dict(c, k=c["k"].copy(), v=c["v"].copy())
+    c2["k"][:, :, 3840:] = rng.integers(-127, 128, c2["k"][:, :, 3840:].shape, dtype=np.int8)
+    c2["v"][:, :, 3840:] = 127
+    assert np.array_equal(gpu_run(pkg, dev, c2), base)
+    # 3840 = 30 whole blocks: the first 3840 query rows equal the 3840-long unmasked problem
+    short = dict(c, q=c["q"][:, :, :3840], k=c["k"][:, :, :3840], v=c["v"][:, :, :3840],
+                 mask=np.zeros((1, 3840), np.int8))
+    assert np.array_equal(gpu_run(pkg, dev, short), base[:, :, :3840])
+
+
+# ---- edge cases ------------------------------------------------------------------------------------------------------
+def test_all_masked_rows_give_zero_and_literal_all_ones_mask(pkg, orc, dev):
+    c = fc.make_inputs(2, 2, 256, 64, seed=41, valid_lengths=[0, 256])
+    got = gpu_run(pkg, dev, c)
+    assert not got[0].any()
+    check(got, cpu_run(orc, c), "batch 0 fully masked")
+    ones = dict(c, mask=np.ones((2, 256), np.int8))  # "all ones" under the reference polarity masks everything
+    assert not gpu_run(pkg, dev, ones).any()
+
+
+@pytest.mark.parametrize("d", [64, 128])
+def test_ragged_and_scattered_masks(pkg, orc, dev, d):
+    # valid lengths that cut blocks at every kind of boundary, one key only, a hole in the middle, non-{0,1} bytes
+    lens = [1, 127, 128, 129, 255, 300, 511, 512]
+    c = fc.make_inputs(len(lens), 2, 512, d, seed=42, valid_lengths=lens)
+    check(gpu_run(pkg, dev, c), cpu_run(orc, c), "ragged d=%d" % d)
+    c = fc.make_inputs(3, 2, 512, d, seed=43, pad="scatter")
+    c["mask"][1, 128:384] = 1          # two whole interior blocks masked
+    c["mask"][2, :128] = 1             # the FIRST block fully masked (the reference kernel yields NaN here)
+    c["mask"] = (c["mask"] * np.int8(-7)).astype(np.int8)  # any nonzero byte masks (inc/fmha_i8.cuh:191)
+    check(gpu_run(pkg, dev, c), cpu_run(orc, c), "scattered d=%d" % d)
+
+
+def test_unaligned_mask_pointer(pkg, orc, dev):
+    import torch
+    c = fc.make_inputs(1, 2, 256, 64, seed=44, valid_lengths=[200])
+    q, k, v = to_dev(dev, c["q"], c["k"], c["v"])
+    buf = torch.zeros(256 + 3, dtype=torch.int8, device=dev)
+    buf[3:] = torch.from_numpy(c["mask"][0]).to(dev)
+    o = torch.empty_like(q)
+    st = pkg.FMHAInferI8Status(None, pkg.FMHAParamI8(c["q_amax"], c["k_amax"], c["v_amax"], 1.0),
+                               pkg.AttnDataDescriptor(1, 256, 2, 64), q, k, v, buf.data_ptr() + 3, o, True)
+    torch.cuda.synchronize()
+    assert st == 0
+    check(o.cpu().numpy(), cpu_run(orc, c), "mask at odd address")
+
+
+def test_saturation_and_clamp(pkg, orc, dev):
+    # heavy tails and v_amax > o_amax: a visible share of O sits at +-127 on both sides
+    c = fc.make_inputs(2, 2, 384, 128, dist="student_t", sigma=0.5, seed=45)
+    want = cpu_run(orc, c, v_amax=4 * c["v_amax"])
+    assert (np.abs(want) == 127).mean() > 0.02
+    check(gpu_run(pkg, dev, c, v_amax=4 * c["v_amax"]), want, "saturating")
+
+
+def test_masked_sentinel_corner(pkg, orc, dev):
+    # every unmasked score of a partially masked block lies below the -1,000,000 substituted for masked keys
+    S, d = 128, 128
+    rng = np.random.default_rng(46)
+    q = np.full((1, 1, S, d), 127, np.int8)
+    k = np.full((1, 1, S, d), -127, np.int8)
+    k[0, 0, ::2, :64] = -100
+    v = rng.integers(-127, 128, (1, 1, S, d), dtype=np.int8)
+    mask = np.zeros((1, S), np.int8)
+    mask[0, 100:] = 1
+    a = float(np.sqrt(0.18))
+    c = dict(q=q, k=k, v=v, mask=mask, q_amax=a, k_amax=a, v_amax=1.0, o_amax=1.0)
+    check(gpu_run(pkg, dev, c), cpu_run(orc, c), "sentinel")
+
+
+def test_one_hot_attention_closed_form_on_gpu(pkg, dev):
+    S = d = 128
+    rng = np.random.default_rng(47)
+    perm = rng.permutation(d)
+    k = np.zeros((1, 1, S, d), np.int8)
+    q = np.zeros((1, 1, S, d), np.int8)
+    k[0, 0, np.arange(S), np.arange(S)] = 127
+    q[0, 0, np.arange(S), perm] = 127
+    v = rng.integers(-127, 128, (1, 1, S, d), dtype=np.int8)
+    c = dict(q=q, k=k, v=v, mask=np.zeros((1, S), np.int8), q_amax=30.0, k_amax=30.0, v_amax=2.0, o_amax=1.0)
+    want = np.clip(2 * v[0, 0, perm].astype(np.int64), -127, 127)
+    assert np.array_equal(gpu_run(pkg, dev, c)[0, 0], want)
+
+
+# ---- API behaviour -----------------------------------------------------------------------------------------------------
+def test_void_entry_point_streams_and_use_tcu_flag(pkg, orc, dev):
+    import torch
+    c = fc.make_inputs(2, 2, 256, 128, seed=48, valid_lengths=[256, 100])
+    q, k, v, m = to_dev(dev, c["q"], c["k"], c["v"], c["mask"])
+    want = cpu_run(orc, c)
+    P = pkg.FMHAParamI8(c["q_amax"], c["k_amax"], c["v_amax"], c["o_amax"], 123.0)  # s_max is ignored
+    A = pkg.AttnDataDescriptor(2, 256, 2, 128)
+    side = torch.cuda.Stream(device=dev)
+    for use_tcu, stream in ((True, None), (False, side)):
+        o = torch.zeros_like(q)
+        if stream is not None:
+            stream.wait_stream(torch.cuda.current_stream(dev))
+        pkg.FMHAInferI8(stream, P, A, q, k, v, m, o, use_tcu)  # the reference's signature: returns nothing
+        torch.cuda.synchronize()
+        check(o.cpu().numpy(), want, "void entry use_tcu=%s" % use_tcu)
+
+
+def test_unsupported_shapes_leave_output_untouched(pkg, dev):
+    import torch
+    q = torch.zeros(1, 1, 192, 64, dtype=torch.int8, device=dev)
+    m = torch.zeros(1, 192, dtype=torch.int8, device=dev)
+    o = torch.full_like(q, 55)
+    P = pkg.FMHAParamI8(1, 1, 1, 1)
+    assert pkg.FMHAInferI8Status(None, P, pkg.AttnDataDescriptor(1, 192, 1, 64), q, q, q, m, o) == \
+        pkg.FMHA_I8_ERR_SEQ_LEN
+    pkg.FMHAInferI8(None, P, pkg.AttnDataDescriptor(1, 128, 1, 96), q, q, q, m, o, True)  # prints, launches nothing
+    torch.cuda.synchronize()
+    assert bool((o == 55).all())
+    with pytest.raises(pkg.FMHAError):
+        pkg.fmha_infer_i8(q, q, q, m, 1.0, 1.0, 1.0)
+
+
+# ---- the C++ harness (host C++ calling the C ABI the way the reference's driver calls its launch function) -------------
+def test_cpp_harness_config1_and_reference_sweep(tmp_path):
+    import json
+    import subprocess
+    exe = os.path.join(HERE, "bin", "test_fmha_i8")
+    assert os.path.exists(exe), "tests/bin/test_fmha_i8 is not built (python -c 'import __graft_entry__ as g; g.build()')"
+    js = str(tmp_path / "harness.json")
+    r = subprocess.run([exe, "--config", "1", "--sweep", "--iters", "20", "--cpu-heads", "0", "--json", js],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+    print(r.stdout[-3000:])
+    assert r.returncode == 0
+    recs = [json.loads(l) for l in open(js)]
+    assert len(recs) == 15 and all(x["pass"] for x in recs)
+    assert all(x["mean_rel_dev_pct"] < 20.0 for x in recs if x["case"] == "sweep")
