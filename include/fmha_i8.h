@@ -15,7 +15,7 @@
  *   asynchrony     one kernel is enqueued on `stream`; the call returns immediately and never synchronises.
  *   threading      no mutable global state: callable concurrently from any host thread.
  *
- * Supported shapes: head_dim in {64, 128}; seq_len a positive multiple of 128; batch_num, head_num >= 1.
+ * Supported shapes: head_dim in {64, 128}; seq_len a positive multiple of 128, at most 65536; batch_num, head_num >= 1.
  * (The reference's ladder, src/fmha_i8.cu:39-154, covers head_dim in {64,128} and eleven fixed seq_len values;
  * every one of its 128-multiples is covered here, and so is any other multiple of 128.)
  *
@@ -38,7 +38,7 @@ extern "C" {
 #define FMHA_I8_OK 0
 #define FMHA_I8_ERR_NULL_POINTER 1   /* q, k, v, padding_mask or o is NULL */
 #define FMHA_I8_ERR_HEAD_DIM 2       /* head_dim not in {64, 128} */
-#define FMHA_I8_ERR_SEQ_LEN 3        /* seq_len <= 0 or not a multiple of 128 */
+#define FMHA_I8_ERR_SEQ_LEN 3        /* seq_len <= 0, not a multiple of 128, or > 65536 */
 #define FMHA_I8_ERR_BATCH_HEAD 4     /* batch_num or head_num <= 0, or the grid would exceed HIP limits */
 #define FMHA_I8_ERR_ALIGNMENT 5      /* q, k, v or o not 16-byte aligned */
 #define FMHA_I8_ERR_SCALE 6          /* an amax is not finite, or o_amax <= 0 */

@@ -17,7 +17,9 @@ int check_args(const FMHAParamI8& p, const AttnDataDescriptor& a, const void* q,
                const void* mask, const void* o) {
   if (!q || !k || !v || !mask || !o) return FMHA_I8_ERR_NULL_POINTER;
   if (a.head_dim != 64 && a.head_dim != 128) return FMHA_I8_ERR_HEAD_DIM;
-  if (a.seq_len <= 0 || a.seq_len % fmha_i8_gfx950::kBlockK != 0) return FMHA_I8_ERR_SEQ_LEN;
+  if (a.seq_len <= 0 || a.seq_len % fmha_i8_gfx950::kBlockK != 0 ||
+      a.seq_len > fmha_i8_gfx950::kBlockK * fmha_i8_gfx950::kMaxKeyBlocks)
+    return FMHA_I8_ERR_SEQ_LEN;
   if (a.batch_num <= 0 || a.head_num <= 0) return FMHA_I8_ERR_BATCH_HEAD;
   const long long wgs = (long long)a.batch_num * a.head_num * (a.seq_len / fmha_i8_gfx950::kBlockQ);
   if (wgs > 0x7fffffffLL) return FMHA_I8_ERR_BATCH_HEAD;
@@ -51,10 +53,18 @@ int launch(hipStream_t stream, const FMHAParamI8& p, const AttnDataDescriptor& a
   args.masked2 = -1000000.f * args.c2;
   args.out_scale = p.v_amax / (p.o_amax * 128.f);  // inc/fmha_i8.cuh:318
   const dim3 grid((unsigned)args.total_wgs), block(fmha_i8_gfx950::kThreads);
-  if (a.head_dim == 128)
-    hipLaunchKernelGGL(fmha_i8_gfx950::fmha_i8_fwd_kernel<128>, grid, block, 0, stream, args);
-  else
-    hipLaunchKernelGGL(fmha_i8_gfx950::fmha_i8_fwd_kernel<64>, grid, block, 0, stream, args);
+  // The accumulators of Q.K^T can be read as floats without a convert when they start at the bit pattern of 1.5*2^23;
+  // the price is that the exponent offset (1.5*2^23 + S)*c2 is then rounded on a coarser float grid.  Take that path
+  // only while the offset stays below 2^12, i.e. while the rounding moves a whole row by less than 2^-13 in log2.
+  const bool bias = (fmha_i8_gfx950::kMagic + 4194304.f) * fabsf(args.c2) < fmha_i8_gfx950::kBiasOffsetLimit;
+  using namespace fmha_i8_gfx950;
+  if (a.head_dim == 128) {
+    if (bias) hipLaunchKernelGGL((fmha_i8_fwd_kernel<128, true>), grid, block, 0, stream, args);
+    else hipLaunchKernelGGL((fmha_i8_fwd_kernel<128, false>), grid, block, 0, stream, args);
+  } else {
+    if (bias) hipLaunchKernelGGL((fmha_i8_fwd_kernel<64, true>), grid, block, 0, stream, args);
+    else hipLaunchKernelGGL((fmha_i8_fwd_kernel<64, false>), grid, block, 0, stream, args);
+  }
   const hipError_t err = hipGetLastError();
   return err == hipSuccess ? FMHA_I8_OK : FMHA_I8_ERR_HIP_BASE + (int)err;
 }
@@ -87,7 +97,7 @@ const char* FMHAInferI8StatusString(int status) {
     case FMHA_I8_OK: return "ok";
     case FMHA_I8_ERR_NULL_POINTER: return "null pointer argument";
     case FMHA_I8_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
-    case FMHA_I8_ERR_SEQ_LEN: return "seq_len must be a positive multiple of 128";
+    case FMHA_I8_ERR_SEQ_LEN: return "seq_len must be a positive multiple of 128, at most 65536";
     case FMHA_I8_ERR_BATCH_HEAD: return "batch_num and head_num must be positive (and the grid must fit)";
     case FMHA_I8_ERR_ALIGNMENT: return "q, k, v and o must be 16-byte aligned";
     case FMHA_I8_ERR_SCALE: return "amax values must be finite and o_amax > 0";
@@ -97,6 +107,6 @@ const char* FMHAInferI8StatusString(int status) {
   return "unknown status";
 }
 
-const char* FMHAInferI8Version(void) { return "fmha_i8 gfx950 mfma32x32x32-lds-swizzle"; }
+const char* FMHAInferI8Version(void) { return "fmha_i8 gfx950 mfma32x32x32 direct-to-lds sdwa-pack"; }
 
 }  // extern "C"
