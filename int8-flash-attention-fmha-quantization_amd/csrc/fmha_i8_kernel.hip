@@ -66,35 +66,63 @@ __device__ __forceinline__ int v_swizzle(int key) {
   return D == 128 ? ((key & 3) | ((key >> 1) & 4)) : (((key >> 1) & 1) | ((key >> 2) & 2));
 }
 
-// dst.byte[BYTE] = low byte of (hi - lo) as float bits; the other bytes of dst are kept (BYTE 0 clears them instead).
-// With hi = 1.5*2^23 and 0 <= lo <= 128 the low byte is the two's-complement int8 of -rne(lo).
-#define FMHA_SDWA_SUB_BYTE(dst, hi, lo, BYTE, UNUSED)                                                            \
-  asm("v_sub_f32_sdwa %0, %1, %2 dst_sel:BYTE_" #BYTE " dst_unused:" UNUSED " src0_sel:DWORD src1_sel:DWORD"     \
-      : "+v"(dst)                                                                                                \
-      : "v"(hi), "v"(lo))
-#define FMHA_SDWA_SUB_BYTE0(dst, hi, lo)                                                                          \
-  asm("v_sub_f32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD"             \
-      : "=v"(dst)                                                                                                \
-      : "v"(hi), "v"(lo))
-#define FMHA_SDWA_ADD_BYTE0(dst, a, b)                                                                           \
-  asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD"             \
-      : "=v"(dst)                                                                                                \
-      : "v"(a), "v"(b))
-#define FMHA_SDWA_ADD_BYTE(dst, a, b, BYTE, UNUSED)                                                              \
-  asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_" #BYTE " dst_unused:" UNUSED " src0_sel:DWORD src1_sel:DWORD"     \
-      : "+v"(dst)                                                                                                \
-      : "v"(a), "v"(b))
-
-__device__ __forceinline__ float max3f(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
+// e_i = 2^x_i for eight exponents, and two words wa, wb holding the bytes -rne(e_i) (two's complement): wa packs
+// e0..e3, wb packs e4..e7.  One block of sixteen instructions with fixed spacing, because the compiler does not track
+// hazards through inline assembly and gfx950 needs (a) one wait state between a transcendental and a VALU use of its
+// result and (b) one wait state between an SDWA write with dst_sel != DWORD and the next read of that register - which
+// includes the next UNUSED_PRESERVE write to it.  The two words are therefore filled alternately.
+#define FMHA_SDWA_TAIL "src0_sel:DWORD src1_sel:DWORD"
+__device__ __forceinline__ void exp2_pack8(const float (&x)[8], float magic, float (&e)[8], int& wa, int& wb) {
+  asm("v_exp_f32 %2, %10\n\t"
+      "v_exp_f32 %3, %11\n\t"
+      "v_exp_f32 %4, %12\n\t"
+      "v_exp_f32 %5, %13\n\t"
+      "v_exp_f32 %6, %14\n\t"
+      "v_exp_f32 %7, %15\n\t"
+      "v_exp_f32 %8, %16\n\t"
+      "v_exp_f32 %9, %17\n\t"
+      "v_sub_f32_sdwa %0, %18, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD " FMHA_SDWA_TAIL "\n\t"
+      "v_sub_f32_sdwa %1, %18, %6 dst_sel:BYTE_0 dst_unused:UNUSED_PAD " FMHA_SDWA_TAIL "\n\t"
+      "v_sub_f32_sdwa %0, %18, %3 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
+      "v_sub_f32_sdwa %1, %18, %7 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
+      "v_sub_f32_sdwa %0, %18, %4 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
+      "v_sub_f32_sdwa %1, %18, %8 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
+      "v_sub_f32_sdwa %0, %18, %5 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
+      "v_sub_f32_sdwa %1, %18, %9 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL
+      : "=&v"(wa), "=&v"(wb), "=&v"(e[0]), "=&v"(e[1]), "=&v"(e[2]), "=&v"(e[3]), "=&v"(e[4]), "=&v"(e[5]),
+        "=&v"(e[6]), "=&v"(e[7])
+      : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "v"(x[4]), "v"(x[5]), "v"(x[6]), "v"(x[7]), "v"(magic));
 }
-__device__ __forceinline__ int max3i(int a, int b, int c) {
-  int r;
-  asm("v_max3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
+// Same packing for values that are already computed (f = +1: bytes of rne(y); f = -1: bytes of -rne(y)).
+template <bool NEG>
+__device__ __forceinline__ void pack8(const float (&y)[8], float magic, int& wa, int& wb) {
+  if (NEG)
+    asm("v_sub_f32_sdwa %0, %10, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD " FMHA_SDWA_TAIL "\n\t"
+        "v_sub_f32_sdwa %1, %10, %6 dst_sel:BYTE_0 dst_unused:UNUSED_PAD " FMHA_SDWA_TAIL "\n\t"
+        "v_sub_f32_sdwa %0, %10, %3 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
+        "v_sub_f32_sdwa %1, %10, %7 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
+        "v_sub_f32_sdwa %0, %10, %4 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
+        "v_sub_f32_sdwa %1, %10, %8 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
+        "v_sub_f32_sdwa %0, %10, %5 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
+        "v_sub_f32_sdwa %1, %10, %9 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL
+        : "=&v"(wa), "=&v"(wb)
+        : "v"(y[0]), "v"(y[1]), "v"(y[2]), "v"(y[3]), "v"(y[4]), "v"(y[5]), "v"(y[6]), "v"(y[7]), "v"(magic));
+  else
+    asm("v_add_f32_sdwa %0, %10, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD " FMHA_SDWA_TAIL "\n\t"
+        "v_add_f32_sdwa %1, %10, %6 dst_sel:BYTE_0 dst_unused:UNUSED_PAD " FMHA_SDWA_TAIL "\n\t"
+        "v_add_f32_sdwa %0, %10, %3 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
+        "v_add_f32_sdwa %1, %10, %7 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
+        "v_add_f32_sdwa %0, %10, %4 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
+        "v_add_f32_sdwa %1, %10, %8 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
+        "v_add_f32_sdwa %0, %10, %5 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
+        "v_add_f32_sdwa %1, %10, %9 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL
+        : "=&v"(wa), "=&v"(wb)
+        : "v"(y[0]), "v"(y[1]), "v"(y[2]), "v"(y[3]), "v"(y[4]), "v"(y[5]), "v"(y[6]), "v"(y[7]), "v"(magic));
 }
+// A VGPR written by an SDWA instruction inside inline assembly and read by an MFMA needs wait states that the compiler
+// only inserts for definitions it can see; this carries the register through four idle issue cycles.
+__device__ __forceinline__ void settle(v4i& x) { asm volatile("s_nop 3" : "+v"(x)); }
+__device__ __forceinline__ void settle(int& x) { asm volatile("s_nop 3" : "+v"(x)); }
 
 // Lanes l and l^32 hold the two halves of one query column: v_permlane32_swap hands each lane both halves.
 __device__ __forceinline__ float half_max(float x) {
@@ -269,23 +297,17 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     float m_blk;        // block-local row maximum, base-2 units
     float l_blk = 0.f;  // sum of 128*p over this lane's keys
     if (cls == 0) {
-      float top;
+      // integer maximum (monotone in the score, also for the biased bit patterns), two independent chains
       constexpr int kVals = 16 * kKeyTiles;  // scores per lane; v(n) = acc[n / 16][n % 16]
-      if (BIAS) {
-        top = __int_as_float(acc[0][0]);
+      int t0 = acc[0][0], t1 = acc[0][1];
 #pragma unroll
-        for (int n = 1; n + 1 < kVals; n += 2)
-          top = max3f(top, __int_as_float(acc[n / 16][n % 16]), __int_as_float(acc[(n + 1) / 16][(n + 1) % 16]));
-        top = fmaxf(top, __int_as_float(acc[kKeyTiles - 1][15]));
-        top = half_max(top);
-      } else {
-        int ti = acc[0][0];
-#pragma unroll
-        for (int n = 1; n + 1 < kVals; n += 2) ti = max3i(ti, acc[n / 16][n % 16], acc[(n + 1) / 16][(n + 1) % 16]);
-        ti = max(ti, acc[kKeyTiles - 1][15]);
-        ti = half_max(ti);
-        top = (float)ti;
+      for (int n = 2; n + 3 < kVals; n += 4) {
+        t0 = max(max(t0, acc[n / 16][n % 16]), acc[(n + 1) / 16][(n + 1) % 16]);
+        t1 = max(max(t1, acc[(n + 2) / 16][(n + 2) % 16]), acc[(n + 3) / 16][(n + 3) % 16]);
       }
+      t0 = max(max(t0, acc[kKeyTiles - 1][14]), acc[kKeyTiles - 1][15]);
+      const int ti = half_max(max(t0, t1));
+      const float top = BIAS ? __int_as_float(ti) : (float)ti;
       // off = top*c2 rounded; p' = exp2(s*c2 - off) = p * 2^(resid) with one row-wide resid below 1 ulp of off, and the
       // block maximum that is consistent with p' is off itself (minus the constant kMagic*c2 when BIAS).
       float off = top * c2;
@@ -295,21 +317,15 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #pragma unroll
       for (int t = 0; t < kKeyTiles; ++t)
 #pragma unroll
-        for (int a = 0; a < 4; ++a) {
-          int w;
-          const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, 4 * a + 0), c2, -off7));
-          const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, 4 * a + 1), c2, -off7));
-          const float e2 = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, 4 * a + 2), c2, -off7));
-          const float e3 = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, 4 * a + 3), c2, -off7));
-          l_blk += e0;
-          l_blk += e1;
-          l_blk += e2;
-          l_blk += e3;
-          FMHA_SDWA_SUB_BYTE0(w, magic, e0);
-          FMHA_SDWA_SUB_BYTE(w, magic, e1, 1, "UNUSED_PRESERVE");
-          FMHA_SDWA_SUB_BYTE(w, magic, e2, 2, "UNUSED_PRESERVE");
-          FMHA_SDWA_SUB_BYTE(w, magic, e3, 3, "UNUSED_PRESERVE");
-          pk[t][a] = w;
+        for (int a = 0; a < 4; a += 2) {
+          float x[8], e[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) x[j] = __builtin_fmaf(sf(t, 4 * a + j), c2, -off7);
+          int wa, wb;
+          exp2_pack8(x, magic, e, wa, wb);
+          pk[t][a] = wa;
+          pk[t][a + 1] = wb;
+          l_blk += ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
         }
     } else {
       // some keys of this block are masked out (nonzero mask byte, inc/fmha_i8.cuh:189-192,216-221)
@@ -335,24 +351,25 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #pragma unroll
       for (int t = 0; t < kKeyTiles; ++t)
 #pragma unroll
-        for (int a = 0; a < 4; ++a) {
-          int w;
-          float e[4];
+        for (int a = 0; a < 4; a += 2) {
+          float e[8];
 #pragma unroll
-          for (int bb = 0; bb < 4; ++bb) {
-            const int r = 4 * a + bb;
+          for (int j = 0; j < 8; ++j) {
+            const int r = 4 * a + j;
             const float ex = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, r), c2, -off7));
-            e[bb] = ((mbits[t] >> r) & 1) ? 0.f : fminf(ex, 128.f);
-            l_blk += e[bb];
+            e[j] = ((mbits[t] >> r) & 1) ? 0.f : fminf(ex, 128.f);
+            l_blk += e[j];
           }
-          FMHA_SDWA_SUB_BYTE0(w, magic, e[0]);
-          FMHA_SDWA_SUB_BYTE(w, magic, e[1], 1, "UNUSED_PRESERVE");
-          FMHA_SDWA_SUB_BYTE(w, magic, e[2], 2, "UNUSED_PRESERVE");
-          FMHA_SDWA_SUB_BYTE(w, magic, e[3], 3, "UNUSED_PRESERVE");
-          pk[t][a] = w;
+          asm volatile("s_nop 0" : "+v"(e[7]));  // keep a wait state between the last exp and the packing block
+          int wa, wb;
+          pack8<true>(e, magic, wa, wb);
+          pk[t][a] = wa;
+          pk[t][a + 1] = wb;
         }
     }
     l_blk = half_sum(l_blk);
+#pragma unroll
+    for (int t = 0; t < kKeyTiles; ++t) settle(pk[t]);
 
     // ---- GEMM 2: O~^T[d][query] = V^T . P^T, int32 (inc/fmha_i8.cuh:255-296); accumulators start at kMagicBits ----
     v16i oacc[kDSteps];
@@ -398,16 +415,16 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #pragma unroll
   for (int u = 0; u < kDSteps; ++u)
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      int w;
-      float y[4];
+    for (int a = 0; a < 4; a += 2) {
+      float y[8];
+      int wa, wb;
 #pragma unroll
-      for (int bb = 0; bb < 4; ++bb) y[bb] = __builtin_amdgcn_fmed3f(o_f[u][4 * a + bb] * fin, -127.f, 127.f);
-      FMHA_SDWA_ADD_BYTE0(w, magic, y[0]);  // round-half-even into the low mantissa byte
-      FMHA_SDWA_ADD_BYTE(w, magic, y[1], 1, "UNUSED_PRESERVE");
-      FMHA_SDWA_ADD_BYTE(w, magic, y[2], 2, "UNUSED_PRESERVE");
-      FMHA_SDWA_ADD_BYTE(w, magic, y[3], 3, "UNUSED_PRESERVE");
-      *reinterpret_cast<int*>(op + 32 * u + 8 * a) = w;
+      for (int j = 0; j < 8; ++j) y[j] = __builtin_amdgcn_fmed3f(o_f[u][4 * a + j] * fin, -127.f, 127.f);
+      pack8<false>(y, magic, wa, wb);  // round-half-even into the low mantissa byte
+      settle(wa);
+      settle(wb);
+      *reinterpret_cast<int*>(op + 32 * u + 8 * a) = wa;
+      *reinterpret_cast<int*>(op + 32 * u + 8 * a + 8) = wb;
     }
 }
 
