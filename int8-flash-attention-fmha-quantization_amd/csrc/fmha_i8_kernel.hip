@@ -37,6 +37,7 @@ constexpr int kMaxKeyBlocks = 512;       // seq_len <= 65536
 constexpr float kMagic = 12582912.0f;    // 1.5 * 2^23: float whose low mantissa bits hold a small signed integer
 constexpr int kMagicBits = 0x4B400000;   // its bit pattern; kMagicBits + n is the float kMagic + n for |n| < 2^22
 constexpr float kBiasOffsetLimit = 4096.0f;  // see the launch code: bound on the exponent offset of the biased path
+constexpr float kLog2Pscale = -7.99995597f;  // log2(128 / 32767): exp2(x + kLog2Pscale) = 128 p / 32767
 constexpr float kLazyLog2 = 10.0f;       // the running O is rescaled only when a row maximum grows by more than this
 
 struct KernelArgs {
@@ -66,63 +67,16 @@ __device__ __forceinline__ int v_swizzle(int key) {
   return D == 128 ? ((key & 3) | ((key >> 1) & 4)) : (((key >> 1) & 1) | ((key >> 2) & 2));
 }
 
-// e_i = 2^x_i for eight exponents, and two words wa, wb holding the bytes -rne(e_i) (two's complement): wa packs
-// e0..e3, wb packs e4..e7.  One block of sixteen instructions with fixed spacing, because the compiler does not track
-// hazards through inline assembly and gfx950 needs (a) one wait state between a transcendental and a VALU use of its
-// result and (b) one wait state between an SDWA write with dst_sel != DWORD and the next read of that register - which
-// includes the next UNUSED_PRESERVE write to it.  The two words are therefore filled alternately.
-#define FMHA_SDWA_TAIL "src0_sel:DWORD src1_sel:DWORD"
-__device__ __forceinline__ void exp2_pack8(const float (&x)[8], float magic, float (&e)[8], int& wa, int& wb) {
-  asm("v_exp_f32 %2, %10\n\t"
-      "v_exp_f32 %3, %11\n\t"
-      "v_exp_f32 %4, %12\n\t"
-      "v_exp_f32 %5, %13\n\t"
-      "v_exp_f32 %6, %14\n\t"
-      "v_exp_f32 %7, %15\n\t"
-      "v_exp_f32 %8, %16\n\t"
-      "v_exp_f32 %9, %17\n\t"
-      "v_sub_f32_sdwa %0, %18, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD " FMHA_SDWA_TAIL "\n\t"
-      "v_sub_f32_sdwa %1, %18, %6 dst_sel:BYTE_0 dst_unused:UNUSED_PAD " FMHA_SDWA_TAIL "\n\t"
-      "v_sub_f32_sdwa %0, %18, %3 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
-      "v_sub_f32_sdwa %1, %18, %7 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
-      "v_sub_f32_sdwa %0, %18, %4 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
-      "v_sub_f32_sdwa %1, %18, %8 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
-      "v_sub_f32_sdwa %0, %18, %5 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
-      "v_sub_f32_sdwa %1, %18, %9 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL
-      : "=&v"(wa), "=&v"(wb), "=&v"(e[0]), "=&v"(e[1]), "=&v"(e[2]), "=&v"(e[3]), "=&v"(e[4]), "=&v"(e[5]),
-        "=&v"(e[6]), "=&v"(e[7])
-      : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "v"(x[4]), "v"(x[5]), "v"(x[6]), "v"(x[7]), "v"(magic));
+// Four floats y_i in [-1, 1] -> four int8 bytes rne(32767 * y_i), packed in order.  v_cvt_pknorm_i16_f32 converts two at a
+// time (round to nearest; exact .5 ties toward zero, which real softmax values do not hit), v_perm_b32 keeps the low
+// byte of each 16-bit result.
+typedef short v2s __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ int pack4_snorm(float y0, float y1, float y2, float y3) {
+  const v2s lo = __builtin_amdgcn_cvt_pknorm_i16(y0, y1);
+  const v2s hi = __builtin_amdgcn_cvt_pknorm_i16(y2, y3);
+  return __builtin_amdgcn_perm(__builtin_bit_cast(int, hi), __builtin_bit_cast(int, lo), 0x06040200);
 }
-// Same packing for values that are already computed (f = +1: bytes of rne(y); f = -1: bytes of -rne(y)).
-template <bool NEG>
-__device__ __forceinline__ void pack8(const float (&y)[8], float magic, int& wa, int& wb) {
-  if (NEG)
-    asm("v_sub_f32_sdwa %0, %10, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD " FMHA_SDWA_TAIL "\n\t"
-        "v_sub_f32_sdwa %1, %10, %6 dst_sel:BYTE_0 dst_unused:UNUSED_PAD " FMHA_SDWA_TAIL "\n\t"
-        "v_sub_f32_sdwa %0, %10, %3 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
-        "v_sub_f32_sdwa %1, %10, %7 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
-        "v_sub_f32_sdwa %0, %10, %4 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
-        "v_sub_f32_sdwa %1, %10, %8 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
-        "v_sub_f32_sdwa %0, %10, %5 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
-        "v_sub_f32_sdwa %1, %10, %9 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL
-        : "=&v"(wa), "=&v"(wb)
-        : "v"(y[0]), "v"(y[1]), "v"(y[2]), "v"(y[3]), "v"(y[4]), "v"(y[5]), "v"(y[6]), "v"(y[7]), "v"(magic));
-  else
-    asm("v_add_f32_sdwa %0, %10, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD " FMHA_SDWA_TAIL "\n\t"
-        "v_add_f32_sdwa %1, %10, %6 dst_sel:BYTE_0 dst_unused:UNUSED_PAD " FMHA_SDWA_TAIL "\n\t"
-        "v_add_f32_sdwa %0, %10, %3 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
-        "v_add_f32_sdwa %1, %10, %7 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
-        "v_add_f32_sdwa %0, %10, %4 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
-        "v_add_f32_sdwa %1, %10, %8 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
-        "v_add_f32_sdwa %0, %10, %5 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL "\n\t"
-        "v_add_f32_sdwa %1, %10, %9 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE " FMHA_SDWA_TAIL
-        : "=&v"(wa), "=&v"(wb)
-        : "v"(y[0]), "v"(y[1]), "v"(y[2]), "v"(y[3]), "v"(y[4]), "v"(y[5]), "v"(y[6]), "v"(y[7]), "v"(magic));
-}
-// A VGPR written by an SDWA instruction inside inline assembly and read by an MFMA needs wait states that the compiler
-// only inserts for definitions it can see; this carries the register through four idle issue cycles.
-__device__ __forceinline__ void settle(v4i& x) { asm volatile("s_nop 3" : "+v"(x)); }
-__device__ __forceinline__ void settle(int& x) { asm volatile("s_nop 3" : "+v"(x)); }
+constexpr float kSnorm = 32767.0f;
 
 // Lanes l and l^32 hold the two halves of one query column: v_permlane32_swap hands each lane both halves.
 __device__ __forceinline__ float half_max(float x) {
@@ -281,13 +235,26 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     // ---- GEMM 1: S^T[key][query] = K . Q^T, int32 (inc/fmha_i8.cuh:120-172) ---------------------------------------
     v16i acc[kKeyTiles];
     const v16i zero_c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    {
+      // operand reads run one k-step ahead of the MFMAs that consume them
+      v4i ka[2][kKeyTiles];
 #pragma unroll
-    for (int kk = 0; kk < kDSteps; ++kk)
+      for (int t = 0; t < kKeyTiles; ++t) ka[0][t] = *reinterpret_cast<const v4i*>(lds_k + k_read_off[0] + 32 * t * D);
 #pragma unroll
-      for (int t = 0; t < kKeyTiles; ++t) {
-        const v4i a = *reinterpret_cast<const v4i*>(lds_k + k_read_off[kk] + 32 * t * D);
-        acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, qreg[kk], kk == 0 ? (BIAS ? magic_c : zero_c) : acc[t], 0, 0, 0);
+      for (int kk = 0; kk < kDSteps; ++kk) {
+        if (kk + 1 < kDSteps) {
+#pragma unroll
+          for (int t = 0; t < kKeyTiles; ++t)
+            ka[(kk + 1) & 1][t] = *reinterpret_cast<const v4i*>(lds_k + k_read_off[kk + 1] + 32 * t * D);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < kKeyTiles; ++t)
+          acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ka[kk & 1][t], qreg[kk],
+                                                         kk == 0 ? (BIAS ? magic_c : zero_c) : acc[t], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
+    }
     // lane holds, for query column i32, keys 32t + 8a + 4g + bb at acc[t][4a+bb]
 
     // ---- block softmax (inc/fmha_i8.cuh:174-253) -----------------------------------------------------------------
@@ -313,19 +280,17 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       float off = top * c2;
       if (!BIAS) off = fmaxf(off, args.floor2);
       m_blk = off - bias_c2;
-      const float off7 = off - 7.0f;  // exp2(x + 7) = 128 p
+      const float offq = off - kLog2Pscale;  // exp2(x - offq) = 128 p / 32767: the snorm conversion returns rne(128 p)
 #pragma unroll
       for (int t = 0; t < kKeyTiles; ++t)
 #pragma unroll
-        for (int a = 0; a < 4; a += 2) {
-          float x[8], e[8];
-#pragma unroll
-          for (int j = 0; j < 8; ++j) x[j] = __builtin_fmaf(sf(t, 4 * a + j), c2, -off7);
-          int wa, wb;
-          exp2_pack8(x, magic, e, wa, wb);
-          pk[t][a] = wa;
-          pk[t][a + 1] = wb;
-          l_blk += ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+        for (int a = 0; a < 4; ++a) {
+          const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, 4 * a + 0), c2, -offq));
+          const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, 4 * a + 1), c2, -offq));
+          const float e2 = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, 4 * a + 2), c2, -offq));
+          const float e3 = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, 4 * a + 3), c2, -offq));
+          l_blk += (e0 + e1) + (e2 + e3);
+          pk[t][a] = pack4_snorm(-e0, -e1, -e2, -e3);
         }
     } else {
       // some keys of this block are masked out (nonzero mask byte, inc/fmha_i8.cuh:189-192,216-221)
@@ -347,43 +312,54 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         for (int r = 0; r < 16; ++r) top = fmaxf(top, ((mbits[t] >> r) & 1) ? masked_s : sf(t, r) * c2);
       const float off = half_max(top);
       m_blk = off - bias_c2;
-      const float off7 = off - 7.0f;
+      const float offq = off - kLog2Pscale;
 #pragma unroll
       for (int t = 0; t < kKeyTiles; ++t)
 #pragma unroll
-        for (int a = 0; a < 4; a += 2) {
-          float e[8];
+        for (int a = 0; a < 4; ++a) {
+          float e[4];
 #pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const int r = 4 * a + j;
-            const float ex = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, r), c2, -off7));
-            e[j] = ((mbits[t] >> r) & 1) ? 0.f : fminf(ex, 128.f);
-            l_blk += e[j];
+          for (int bb = 0; bb < 4; ++bb) {
+            const int r = 4 * a + bb;
+            const float ex = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, r), c2, -offq));
+            e[bb] = ((mbits[t] >> r) & 1) ? 0.f : ex;
+            l_blk += e[bb];
           }
-          asm volatile("s_nop 0" : "+v"(e[7]));  // keep a wait state between the last exp and the packing block
-          int wa, wb;
-          pack8<true>(e, magic, wa, wb);
-          pk[t][a] = wa;
-          pk[t][a + 1] = wb;
+          pk[t][a] = pack4_snorm(-e[0], -e[1], -e[2], -e[3]);
         }
     }
     l_blk = half_sum(l_blk);
-#pragma unroll
-    for (int t = 0; t < kKeyTiles; ++t) settle(pk[t]);
 
     // ---- GEMM 2: O~^T[d][query] = V^T . P^T, int32 (inc/fmha_i8.cuh:255-296); accumulators start at kMagicBits ----
     v16i oacc[kDSteps];
-#pragma unroll
-    for (int t = 0; t < kKeyTiles; ++t)
+    {
+      typedef v2i __attribute__((address_space(3))) * lds_v2i_ptr;
+      v2i va[2][kDSteps][2];  // transposed V operands, one 32-key tile ahead of the MFMAs
 #pragma unroll
       for (int u = 0; u < kDSteps; ++u) {
-        typedef v2i __attribute__((address_space(3))) * lds_v2i_ptr;
-        const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u] + 32 * t * D));
-        const v2i hi =
-            __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u] + 32 * t * D + 16 * D));
-        const v4i a = {lo[0], lo[1], hi[0], hi[1]};
-        oacc[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, pk[t], t == 0 ? magic_c : oacc[u], 0, 0, 0);
+        va[0][u][0] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u]));
+        va[0][u][1] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u] + 16 * D));
       }
+#pragma unroll
+      for (int t = 0; t < kKeyTiles; ++t) {
+        if (t + 1 < kKeyTiles) {
+#pragma unroll
+          for (int u = 0; u < kDSteps; ++u) {
+            va[(t + 1) & 1][u][0] =
+                __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u] + 32 * (t + 1) * D));
+            va[(t + 1) & 1][u][1] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                (lds_v2i_ptr)(lds_v + v_read_off[u] + 32 * (t + 1) * D + 16 * D));
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < kDSteps; ++u) {
+          const v4i a = {va[t & 1][u][0][0], va[t & 1][u][0][1], va[t & 1][u][1][0], va[t & 1][u][1][1]};
+          oacc[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, pk[t], t == 0 ? magic_c : oacc[u], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
     // lane holds, for query column i32, output dims 32u + 8a + 4g + bb at oacc[u][4a+bb], as the float kMagic + O~
 
     // ---- online merge, normalisation deferred to the epilogue (inc/fmha_i8.cuh:298-315) ---------------------------
@@ -409,22 +385,20 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   }
 
   // ---- epilogue: normalise, requantise, store (inc/fmha_i8.cuh:318-332) --------------------------------------------
-  // l_run sums 128*p, O sums 128*p*v: the two factors of 128 cancel against the 1/128 of out_scale.
-  const float fin = (l_run > 0.f) ? args.out_scale * 128.f / l_run : 0.f;  // a row with no unmasked key yields 0
+  // l_run sums 128 p / 32767 and O sums 128 p v, so mean(v) = O / (32767 l_run); a row with no unmasked key yields 0
+  const float fin = (l_run > 0.f) ? args.out_scale * (128.f / kSnorm) / l_run : 0.f;
   int8_t* op = args.o + head_off + (long)(qb * kBlockQ + wave * 32 + i32) * D + 4 * g;
 #pragma unroll
   for (int u = 0; u < kDSteps; ++u)
 #pragma unroll
-    for (int a = 0; a < 4; a += 2) {
-      float y[8];
-      int wa, wb;
+    for (int a = 0; a < 4; ++a) {
+      float y[4];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) y[j] = __builtin_amdgcn_fmed3f(o_f[u][4 * a + j] * fin, -127.f, 127.f);
-      pack8<false>(y, magic, wa, wb);  // round-half-even into the low mantissa byte
-      settle(wa);
-      settle(wb);
-      *reinterpret_cast<int*>(op + 32 * u + 8 * a) = wa;
-      *reinterpret_cast<int*>(op + 32 * u + 8 * a + 8) = wb;
+      for (int bb = 0; bb < 4; ++bb) y[bb] = __builtin_amdgcn_fmed3f(o_f[u][4 * a + bb] * fin, -127.f, 127.f) + magic;
+      // magic + y holds rne(y) in the low mantissa byte (round-half-even)
+      const int lo = __builtin_amdgcn_perm(__float_as_int(y[1]), __float_as_int(y[0]), 0x0c0c0400);
+      const int hi = __builtin_amdgcn_perm(__float_as_int(y[3]), __float_as_int(y[2]), 0x0c0c0400);
+      *reinterpret_cast<int*>(op + 32 * u + 8 * a) = __builtin_amdgcn_perm(hi, lo, 0x05040100);
     }
 }
 
