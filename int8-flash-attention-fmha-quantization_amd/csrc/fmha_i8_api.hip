@@ -21,7 +21,7 @@ int check_args(const FMHAParamI8& p, const AttnDataDescriptor& a, const void* q,
       a.seq_len > fmha_i8_gfx950::kBlockK * fmha_i8_gfx950::kMaxKeyBlocks)
     return FMHA_I8_ERR_SEQ_LEN;
   if (a.batch_num <= 0 || a.head_num <= 0) return FMHA_I8_ERR_BATCH_HEAD;
-  const long long wgs = (long long)a.batch_num * a.head_num * (a.seq_len / fmha_i8_gfx950::kBlockQ);
+  const long long wgs = (long long)a.batch_num * a.head_num * ((a.seq_len + fmha_i8_gfx950::kBlockQ - 1) / fmha_i8_gfx950::kBlockQ);
   if (wgs > 0x7fffffffLL) return FMHA_I8_ERR_BATCH_HEAD;
   const uintptr_t bits = (uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o;
   if (bits & 15u) return FMHA_I8_ERR_ALIGNMENT;
@@ -43,7 +43,7 @@ int launch(hipStream_t stream, const FMHAParamI8& p, const AttnDataDescriptor& a
   args.o = static_cast<int8_t*>(o);
   args.seq_len = a.seq_len;
   args.head_num = a.head_num;
-  args.q_blocks = a.seq_len / fmha_i8_gfx950::kBlockQ;
+  args.q_blocks = (a.seq_len + fmha_i8_gfx950::kBlockQ - 1) / fmha_i8_gfx950::kBlockQ;
   args.total_wgs = a.batch_num * a.head_num * args.q_blocks;
   // inc/fmha_i8.cuh:71-72: row_scale = 1/sqrt(d), scale_qk_out = q_amax*k_amax/127^2; folded with log2(e).
   const float row_scale = 1.0f / sqrtf((float)a.head_dim);
@@ -107,6 +107,6 @@ const char* FMHAInferI8StatusString(int status) {
   return "unknown status";
 }
 
-const char* FMHAInferI8Version(void) { return "fmha_i8 gfx950 mfma32x32x32 direct-to-lds sdwa-pack"; }
+const char* FMHAInferI8Version(void) { return "fmha_i8 gfx950 mfma32x32x32 direct-to-lds anti-phase"; }
 
 }  // extern "C"

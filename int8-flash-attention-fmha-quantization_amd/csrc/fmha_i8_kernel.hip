@@ -6,20 +6,25 @@
 // online (m, l, O) merge across key blocks, and O requantised to int8 with v_amax/(128*o_amax), clamp +-127.
 //
 // How it computes it is designed for CDNA4, not taken from the reference:
-//   * grid over (query block of 128 rows) x head x batch, XCD-aware so that the query blocks of one head share an L2;
-//     4 wavefronts of 64 lanes per workgroup, each wavefront owns 32 query rows; 2 workgroups per CU;
+//   * grid over (query block of 256 rows) x head x batch, XCD-aware so that the query blocks of one head share an L2;
+//     one workgroup of 8 wavefronts per CU, each wavefront owns 32 query rows, two wavefronts per SIMD;
 //   * both GEMMs run on v_mfma_i32_32x32x32_i8 in the TRANSPOSED formulation S^T = K.Q^T and O^T = V^T.P^T: each
 //     lane then owns one query column, so the row max / row sum are in-register reductions plus one exchange with
 //     lane^32, and the quantised P^T tile leaves the accumulator already in the B-operand register layout;
 //   * K and V tiles of 128 keys go HBM -> LDS directly (global_load_lds_dwordx4, no VGPR staging, no ds_write),
-//     double buffered, as [key][d] with the 16-byte chunk index XOR-swizzled by the row (the swizzle is applied to the
-//     global address each lane fetches), so that the 128-bit operand reads of K and the transposing reads of V
-//     (ds_read_b64_tr_b8) are bank-conflict free; Q goes once per workgroup straight into MFMA operand registers;
-//   * the softmax is written for the VALU issue port, which is what bounds this kernel: exp in the base-2 domain
-//     with every scale folded into one fma, v_max3 for the row maximum, P converted AND packed by one SDWA subtract
-//     per element (magic-number rounding, result byte written in place), the int32 accumulators of both GEMMs start
-//     at the bit pattern of 1.5*2^23 so that they can be read as floats without a convert, the running O is only
-//     rescaled when a row maximum jumps by more than 2^kLazyLog2, and O is normalised once, in the epilogue.
+//     double buffered and fetched two key blocks ahead, as [key][d] with the 16-byte chunk index XOR-swizzled by the
+//     row (the swizzle is applied to the global address each lane fetches), so that the 128-bit operand reads of K and
+//     the transposing reads of V (ds_read_b64_tr_b8) are bank-conflict free; Q goes once per workgroup straight into
+//     MFMA operand registers;
+//   * the kernel is bound by the VALU issue port (a wavefront issues one VALU instruction per ~4.5 cycles), so the
+//     two wavefronts that share a SIMD run in ANTI-PHASE: every key block is four phases - GEMM 1 (MFMA), softmax
+//     (VALU), GEMM 2 (MFMA), merge (VALU) - separated by workgroup barriers, and wavefronts 4..7 run one phase behind
+//     wavefronts 0..3, so an MFMA phase of one always overlaps a VALU phase of the other on the same SIMD;
+//   * the softmax is written for instruction count: exp in the base-2 domain with every scale folded into one fma,
+//     v_max3 on the raw accumulators for the row maximum, P converted two at a time by v_cvt_pknorm_i16_f32 and packed
+//     by v_perm_b32, the int32 accumulators of both GEMMs start at the bit pattern of 1.5*2^23 so that they can be
+//     read as floats without a convert, the running O is only rescaled when a row maximum jumps by more than
+//     2^kLazyLog2, and O is normalised once, in the epilogue.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -29,9 +34,9 @@ typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int kBlockQ = 128;   // query rows per workgroup
+constexpr int kBlockQ = 256;   // query rows per workgroup
 constexpr int kBlockK = 128;   // keys per softmax block (the reference's BASE_SEQ_LEN, src/fmha_i8.cu:61-95)
-constexpr int kThreads = 256;  // 4 wavefronts
+constexpr int kThreads = 512;  // 8 wavefronts: 0..3 and 4..7 run the key-block phases one phase apart
 constexpr int kXcds = 8;
 constexpr int kMaxKeyBlocks = 512;       // seq_len <= 65536
 constexpr float kMagic = 12582912.0f;    // 1.5 * 2^23: float whose low mantissa bits hold a small signed integer
@@ -48,7 +53,7 @@ struct KernelArgs {
   int8_t* o;
   int seq_len;
   int head_num;
-  int q_blocks;     // seq_len / kBlockQ
+  int q_blocks;     // ceil(seq_len / kBlockQ)
   int total_wgs;    // batch * head_num * q_blocks
   float c2;         // log2(e) * (1/sqrt(d)) * q_amax*k_amax/127^2 : int32 S -> base-2 exponent
   float floor2;     // log2(e) * -1e6 : the reference's initial block maximum (inc/fmha_i8.cuh:116)
@@ -98,14 +103,14 @@ template <int D, bool BIAS>
 __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelArgs args) {
   constexpr int kChunks = D / 16;                     // 16-byte chunks per row
   constexpr int kTileBytes = kBlockK * D;             // one K or V tile
-  constexpr int kRegionsPerWave = kTileBytes / 1024 / 4;  // 1 KiB (64 lanes x 16 B) direct-to-LDS loads per wave
+  constexpr int kWaves = kThreads / 64;
+  constexpr int kRegionsPerWave = kTileBytes / 1024 / kWaves;  // 1 KiB (64 lanes x 16 B) direct-to-LDS loads per wave
   constexpr int kRowsPerRegion = 1024 / D;
   constexpr int kDSteps = D / 32;                     // MFMA k-steps of GEMM 1, and 32-row output tiles of GEMM 2
   constexpr int kKeyTiles = kBlockK / 32;
 
   __shared__ __attribute__((aligned(1024))) int8_t lds[2][2][kTileBytes];  // [buffer][K|V][tile]
   __shared__ unsigned char lds_class[kMaxKeyBlocks];  // per key block: bit0 = some key masked, bit1 = all keys masked
-  __shared__ int lds_last_block;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -130,33 +135,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   const int8_t* __restrict__ mg = args.mask + (long)b * S;
   const int n_blocks = S / kBlockK;
 
-  // ---- classify the key blocks of this batch entry: 4 mask bytes per lane, two blocks per wavefront ballot ---------
-  if (tid == 0) lds_last_block = -1;
-  __syncthreads();
-  for (int base = 0; base < S; base += 4 * kThreads) {
-    const int j = base + 4 * tid;
-    int nib = 15;
-    if (j < S) nib = (mg[j] != 0 ? 1 : 0) | (mg[j + 1] != 0 ? 2 : 0) | (mg[j + 2] != 0 ? 4 : 0) | (mg[j + 3] != 0 ? 8 : 0);
-    const unsigned long long some = __ballot(nib != 0), all = __ballot(nib == 15);
-    if ((lane & 31) == 0 && j < S) {
-      const unsigned half_some = (unsigned)(some >> (lane & 32)), half_all = (unsigned)(all >> (lane & 32));
-      const int blk = j / kBlockK;
-      const int cls = (half_some != 0 ? 1 : 0) | (half_all == 0xffffffffu ? 2 : 0);
-      lds_class[blk] = (unsigned char)cls;
-      if (!(cls & 2)) atomicMax(&lds_last_block, blk);
-    }
-  }
-
-  // ---- Q: B operand of GEMM 1, loaded once -----------------------------------------------------------------------
-  v4i qreg[kDSteps];
-  {
-    const int8_t* qp = args.q + head_off + (long)(qb * kBlockQ + wave * 32 + i32) * D + 16 * g;
-#pragma unroll
-    for (int kk = 0; kk < kDSteps; ++kk) qreg[kk] = *reinterpret_cast<const v4i*>(qp + 32 * kk);
-  }
-  __syncthreads();
-  const int kb_end = __builtin_amdgcn_readfirstlane(lds_last_block) + 1;
-
+  // The prologue puts every cold miss in flight before it waits for any of them: the first two K/V tiles (tile 1 on
+  // speculation: it exists whenever seq_len >= 256, whether or not its keys are masked), the Q rows, and the mask bytes.
   // ---- per-lane addressing -----------------------------------------------------------------------------------------
   // direct-to-LDS loads: lane l of a 1 KiB region lands at byte 16*l of the region, so the lane FETCHES the chunk that
   // the swizzle assigns to that slot.
@@ -182,24 +162,68 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   }
 
   // HBM -> LDS without passing through registers.  Written as inline assembly on purpose: the compiler treats an
-  // LDS-DMA builtin as a store that may alias every later LDS read and would wait for the NEXT tile (vmcnt(0)) before
-  // the first operand read of the CURRENT one.  Completion is tracked by hand: s_waitcnt vmcnt(0) + barrier at the top
-  // of each iteration.  M0 carries the LDS destination of lane 0; lane l lands 16*l bytes further.
+  // LDS-DMA builtin as a store that may alias every later LDS read and would wait for tiles that are still in flight
+  // before the first operand read of the current one.  Completion is tracked by hand with s_waitcnt vmcnt(n) in front
+  // of the barrier that publishes a tile.  M0 carries the LDS destination of lane 0; lane l lands 16*l bytes further.
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) int8_t*)&lds[0][0][0];
-  auto issue_tile_loads = [&](int kb, int buf) {
-    const int8_t* kp = kg + (long)kb * kTileBytes;  // wave-uniform bases (SGPR pairs)
-    const int8_t* vp = vg + (long)kb * kTileBytes;
+  auto issue_tile = [&](const int8_t* gbase, int kb, int which, int goff) {  // which: 0 = K, 1 = V
+    const int8_t* gp = gbase + (long)kb * kTileBytes;  // wave-uniform base (SGPR pair)
 #pragma unroll
     for (int it = 0; it < kRegionsPerWave; ++it) {
-      const int region = it * 4 + wave;
-      const unsigned dst_k = lds_base + (unsigned)((buf * 2 + 0) * kTileBytes + region * 1024);
-      const unsigned dst_v = lds_base + (unsigned)((buf * 2 + 1) * kTileBytes + region * 1024);
+      const int region = it * kWaves + wave;
+      const unsigned dst = lds_base + (unsigned)(((kb & 1) * 2 + which) * kTileBytes + region * 1024);
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                   :: "s"(dst_k), "v"(ld_goff_k + region * 1024), "s"(kp) : "memory");
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                   :: "s"(dst_v), "v"(ld_goff_v + region * 1024), "s"(vp) : "memory");
+                   :: "s"(dst), "v"(goff + region * 1024), "s"(gp) : "memory");
     }
   };
+  auto issue_k = [&](int kb) { issue_tile(kg, kb, 0, ld_goff_k); };
+  auto issue_v = [&](int kb) { issue_tile(vg, kb, 1, ld_goff_v); };
+  // Every wavefront issues its loads in the order K0 V0 K1 V1 K2 V2 ..., kRegionsPerWave per tile, and memory reads
+  // return in order: waiting until at most `2 tiles` of this wavefront's loads are outstanding retires everything up to
+  // and including the tile that is two tiles older than the newest one.
+  auto wait_all_but_two_tiles = [&]() {
+    if (kRegionsPerWave == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+  };
+  auto wait_all = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+  auto barrier = [&]() { asm volatile("s_barrier" ::: "memory"); };
+
+  issue_k(0);
+  issue_v(0);
+  if (n_blocks > 1) { issue_k(1); issue_v(1); }
+
+  // ---- Q: B operand of GEMM 1, loaded once -----------------------------------------------------------------------
+  const int row0 = qb * kBlockQ + wave * 32;  // first query row of this wavefront
+  const bool active = row0 < S;               // seq_len is a multiple of 128, not of 256: the last workgroup may be half empty
+  v4i qreg[kDSteps];
+#pragma unroll
+  for (int kk = 0; kk < kDSteps; ++kk) qreg[kk] = v4i{0, 0, 0, 0};
+  if (active) {
+    const int8_t* qp = args.q + head_off + (long)(row0 + i32) * D + 16 * g;
+#pragma unroll
+    for (int kk = 0; kk < kDSteps; ++kk) qreg[kk] = *reinterpret_cast<const v4i*>(qp + 32 * kk);
+  }
+
+  // ---- classify the key blocks of this batch entry: 4 mask bytes per lane, two blocks per wavefront ballot ---------
+  for (int base = 0; base < S; base += 4 * kThreads) {
+    const int j = base + 4 * tid;
+    int nib = 15;
+    if (j < S) nib = (mg[j] != 0 ? 1 : 0) | (mg[j + 1] != 0 ? 2 : 0) | (mg[j + 2] != 0 ? 4 : 0) | (mg[j + 3] != 0 ? 8 : 0);
+    const unsigned long long some = __ballot(nib != 0), all = __ballot(nib == 15);
+    if ((lane & 31) == 0 && j < S) {
+      const unsigned half_some = (unsigned)(some >> (lane & 32)), half_all = (unsigned)(all >> (lane & 32));
+      lds_class[j / kBlockK] = (unsigned char)((half_some != 0 ? 1 : 0) | (half_all == 0xffffffffu ? 2 : 0));
+    }
+  }
+  __syncthreads();
+  // last key block that holds any unmasked key (trailing padding is never computed on)
+  int last_block = -1;
+  for (int base = 0; base < n_blocks; base += 64) {
+    const int blk = base + lane;
+    const unsigned long long live = __ballot(blk < n_blocks && !(lds_class[blk < n_blocks ? blk : 0] & 2));
+    if (live != 0) last_block = base + 63 - __builtin_clzll(live);
+  }
+  const int kb_end = __builtin_amdgcn_readfirstlane(last_block) + 1;
 
   float o_f[kDSteps][16];
 #pragma unroll
@@ -210,7 +234,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   float l_run = 0.f;                            // running row sum, in units of 1/128 (it sums 128*p)
   const float c2 = args.c2;
   const float bias_c2 = BIAS ? kMagic * c2 : 0.f;
-  const float magic = kMagic;
+  float magic = kMagic;
+  asm volatile("" : "+v"(magic));  // a register operand: as a literal it would double the size of every instruction using it
   v16i magic_c;  // C operand that starts an accumulation chain at kMagicBits without per-element moves
 #pragma unroll
   for (int r = 0; r < 16; ++r) magic_c[r] = kMagicBits;
@@ -220,49 +245,41 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // hand-issued LDS-DMA loads and would otherwise wait for them inside the loop.
 #pragma unroll
   for (int kk = 0; kk < kDSteps; ++kk) asm volatile("" ::"v"(qreg[kk]));
-  if (kb_end > 0) issue_tile_loads(0, 0);
 
-  for (int kb = 0; kb < kb_end; ++kb) {
-    const int buf = kb & 1;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();  // tile kb has landed for every wave; every wave is done reading the other buffer
-    if (kb + 1 < kb_end) issue_tile_loads(kb + 1, buf ^ 1);
-    const int cls = __builtin_amdgcn_readfirstlane((int)lds_class[kb]);
-    if (cls & 2) continue;  // nothing in this block is attended to
-    const int8_t* lds_k = &lds[buf][0][0];
-    const int8_t* lds_v = &lds[buf][1][0];
+  // ---- the four phases of one key block ----------------------------------------------------------------------------
+  // acc:  S^T, for query column i32 keys 32t + 8a + 4g + bb at acc[t][4a+bb]        (GEMM 1 -> softmax)
+  // pk:   P^T, int8, B operand of GEMM 2                                              (softmax -> GEMM 2)
+  // oacc: O~^T, output dims 32u + 8a + 4g + bb at oacc[u][4a+bb], as kMagic + O~      (GEMM 2 -> merge)
+  float m_blk = 0.f;    // block-local row maximum, base-2 units
+  float l_blk = 0.f;    // sum of (128/32767) p over this lane's keys
 
-    // ---- GEMM 1: S^T[key][query] = K . Q^T, int32 (inc/fmha_i8.cuh:120-172) ---------------------------------------
-    v16i acc[kKeyTiles];
+  // GEMM 1: S^T[key][query] = K . Q^T, int32 (inc/fmha_i8.cuh:120-172)
+  auto phase_gemm1 = [&](int kb, v16i (&acc)[kKeyTiles]) {
+    const int8_t* lds_k = &lds[kb & 1][0][0];
     const v16i zero_c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    {
-      // operand reads run one k-step ahead of the MFMAs that consume them
-      v4i ka[2][kKeyTiles];
+    v4i ka[2][kKeyTiles];  // operand reads run one k-step ahead of the MFMAs that consume them
 #pragma unroll
-      for (int t = 0; t < kKeyTiles; ++t) ka[0][t] = *reinterpret_cast<const v4i*>(lds_k + k_read_off[0] + 32 * t * D);
+    for (int t = 0; t < kKeyTiles; ++t) ka[0][t] = *reinterpret_cast<const v4i*>(lds_k + k_read_off[0] + 32 * t * D);
 #pragma unroll
-      for (int kk = 0; kk < kDSteps; ++kk) {
-        if (kk + 1 < kDSteps) {
-#pragma unroll
-          for (int t = 0; t < kKeyTiles; ++t)
-            ka[(kk + 1) & 1][t] = *reinterpret_cast<const v4i*>(lds_k + k_read_off[kk + 1] + 32 * t * D);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+    for (int kk = 0; kk < kDSteps; ++kk) {
+      if (kk + 1 < kDSteps) {
 #pragma unroll
         for (int t = 0; t < kKeyTiles; ++t)
-          acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ka[kk & 1][t], qreg[kk],
-                                                         kk == 0 ? (BIAS ? magic_c : zero_c) : acc[t], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
+          ka[(kk + 1) & 1][t] = *reinterpret_cast<const v4i*>(lds_k + k_read_off[kk + 1] + 32 * t * D);
       }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int t = 0; t < kKeyTiles; ++t)
+        acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ka[kk & 1][t], qreg[kk],
+                                                       kk == 0 ? (BIAS ? magic_c : zero_c) : acc[t], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    // lane holds, for query column i32, keys 32t + 8a + 4g + bb at acc[t][4a+bb]
-
-    // ---- block softmax (inc/fmha_i8.cuh:174-253) -----------------------------------------------------------------
-    // sf(t,r): the score as a float; with BIAS it still carries +kMagic, which the exponent offset removes.
+  };
+  // (sf(t,r) below: the score as a float; with BIAS it still carries +kMagic, which the exponent offset removes.)
+  // block softmax (inc/fmha_i8.cuh:174-253)
+  auto phase_softmax = [&](int kb, int cls, const v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles]) {
     auto sf = [&](int t, int r) -> float { return BIAS ? __int_as_float(acc[t][r]) : (float)acc[t][r]; };
-    v4i pk[kKeyTiles];
-    float m_blk;        // block-local row maximum, base-2 units
-    float l_blk = 0.f;  // sum of 128*p over this lane's keys
+    l_blk = 0.f;
     if (cls == 0) {
       // integer maximum (monotone in the score, also for the biased bit patterns), two independent chains
       constexpr int kVals = 16 * kKeyTiles;  // scores per lane; v(n) = acc[n / 16][n % 16]
@@ -281,17 +298,30 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       if (!BIAS) off = fmaxf(off, args.floor2);
       m_blk = off - bias_c2;
       const float offq = off - kLog2Pscale;  // exp2(x - offq) = 128 p / 32767: the snorm conversion returns rne(128 p)
+      // Three stages per 32-key tile - 16 fma, 16 exp, then sums and packing - software-pipelined one tile apart and
+      // fenced for the scheduler, so that every instruction is far from the one whose result it needs: a wavefront
+      // issues in order and a transcendental takes several issue slots to deliver.
+      float e[2][16];
+      auto stage_exp = [&](int t) {
 #pragma unroll
-      for (int t = 0; t < kKeyTiles; ++t)
+        for (int r = 0; r < 16; ++r) e[t & 1][r] = __builtin_fmaf(sf(t, r), c2, -offq);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) e[t & 1][r] = __builtin_amdgcn_exp2f(e[t & 1][r]);
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      stage_exp(0);
+#pragma unroll
+      for (int t = 0; t < kKeyTiles; ++t) {
+        if (t + 1 < kKeyTiles) stage_exp(t + 1);
+        const float(&et)[16] = e[t & 1];
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
-          const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, 4 * a + 0), c2, -offq));
-          const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, 4 * a + 1), c2, -offq));
-          const float e2 = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, 4 * a + 2), c2, -offq));
-          const float e3 = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, 4 * a + 3), c2, -offq));
-          l_blk += (e0 + e1) + (e2 + e3);
-          pk[t][a] = pack4_snorm(-e0, -e1, -e2, -e3);
+          l_blk += (et[4 * a] + et[4 * a + 1]) + (et[4 * a + 2] + et[4 * a + 3]);
+          pk[t][a] = pack4_snorm(-et[4 * a], -et[4 * a + 1], -et[4 * a + 2], -et[4 * a + 3]);
         }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     } else {
       // some keys of this block are masked out (nonzero mask byte, inc/fmha_i8.cuh:189-192,216-221)
       const int8_t* mp = mg + kb * kBlockK + 4 * i32;
@@ -329,41 +359,42 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         }
     }
     l_blk = half_sum(l_blk);
+  };
 
-    // ---- GEMM 2: O~^T[d][query] = V^T . P^T, int32 (inc/fmha_i8.cuh:255-296); accumulators start at kMagicBits ----
-    v16i oacc[kDSteps];
-    {
-      typedef v2i __attribute__((address_space(3))) * lds_v2i_ptr;
-      v2i va[2][kDSteps][2];  // transposed V operands, one 32-key tile ahead of the MFMAs
+  // GEMM 2: O~^T[d][query] = V^T . P^T, int32 (inc/fmha_i8.cuh:255-296); accumulators start at kMagicBits
+  auto phase_gemm2 = [&](int kb, const v4i (&pk)[kKeyTiles], v16i (&oacc)[kDSteps]) {
+    const int8_t* lds_v = &lds[kb & 1][1][0];
+    typedef v2i __attribute__((address_space(3))) * lds_v2i_ptr;
+    v2i va[2][kDSteps][2];  // transposed V operands, one 32-key tile ahead of the MFMAs
 #pragma unroll
-      for (int u = 0; u < kDSteps; ++u) {
-        va[0][u][0] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u]));
-        va[0][u][1] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u] + 16 * D));
-      }
+    for (int u = 0; u < kDSteps; ++u) {
+      va[0][u][0] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u]));
+      va[0][u][1] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u] + 16 * D));
+    }
 #pragma unroll
-      for (int t = 0; t < kKeyTiles; ++t) {
-        if (t + 1 < kKeyTiles) {
-#pragma unroll
-          for (int u = 0; u < kDSteps; ++u) {
-            va[(t + 1) & 1][u][0] =
-                __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u] + 32 * (t + 1) * D));
-            va[(t + 1) & 1][u][1] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-                (lds_v2i_ptr)(lds_v + v_read_off[u] + 32 * (t + 1) * D + 16 * D));
-          }
-        }
-        __builtin_amdgcn_sched_barrier(0);
+    for (int t = 0; t < kKeyTiles; ++t) {
+      if (t + 1 < kKeyTiles) {
 #pragma unroll
         for (int u = 0; u < kDSteps; ++u) {
-          const v4i a = {va[t & 1][u][0][0], va[t & 1][u][0][1], va[t & 1][u][1][0], va[t & 1][u][1][1]};
-          oacc[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, pk[t], t == 0 ? magic_c : oacc[u], 0, 0, 0);
+          va[(t + 1) & 1][u][0] =
+              __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u] + 32 * (t + 1) * D));
+          va[(t + 1) & 1][u][1] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+              (lds_v2i_ptr)(lds_v + v_read_off[u] + 32 * (t + 1) * D + 16 * D));
         }
-        __builtin_amdgcn_sched_barrier(0);
       }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int u = 0; u < kDSteps; ++u) {
+        const v4i a = {va[t & 1][u][0][0], va[t & 1][u][0][1], va[t & 1][u][1][0], va[t & 1][u][1][1]};
+        oacc[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, pk[t], t == 0 ? magic_c : oacc[u], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
-    // lane holds, for query column i32, output dims 32u + 8a + 4g + bb at oacc[u][4a+bb], as the float kMagic + O~
+  };
 
-    // ---- online merge, normalisation deferred to the epilogue (inc/fmha_i8.cuh:298-315) ---------------------------
-    // O and l are kept relative to 2^m_ref; m_ref only moves when some row's block maximum exceeds it by 2^kLazyLog2.
+  // online merge, normalisation deferred to the epilogue (inc/fmha_i8.cuh:298-315).  O and l are kept relative to
+  // 2^m_ref; m_ref only moves when some row's block maximum exceeds it by 2^kLazyLog2.
+  auto phase_merge = [&](const v16i (&oacc)[kDSteps]) {
     if (__ballot(m_blk > m_ref + kLazyLog2) != 0) {
       const float m_new = fmaxf(m_ref, m_blk);
       const float keep = __builtin_amdgcn_exp2f(m_ref - m_new);
@@ -382,12 +413,85 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #pragma unroll
       for (int r = 0; r < 16; ++r)
         o_f[u][r] = __builtin_fmaf(neg_take, __int_as_float(oacc[u][r]) - magic, o_f[u][r]);
+  };
+
+  // ---- the tick schedule -------------------------------------------------------------------------------------------
+  // A tick is the interval between two workgroup barriers.  In tick T wavefronts 0..3 run phase T mod 4 of key block
+  // T div 4 (GEMM 1, softmax, GEMM 2, merge) and wavefronts 4..7 run phase (T-1) mod 4 of block (T-1) div 4.
+  // Tiles: K(j), V(j) live in buffer j mod 2.  K(j) is read in ticks 4j and 4j+1, V(j) in ticks 4j+2 and 4j+3, so
+  // K(j+2) may be fetched after barrier 4j+2 and V(j+2) after barrier 4j+4; every wavefront issues its share in the
+  // order K0 V0 K1 V1 K2 ..., K(j) must have landed before barrier 4j and V(j) before barrier 4j+2.
+  const int n = kb_end;
+  auto cls_of = [&](int kb) { return __builtin_amdgcn_readfirstlane((int)lds_class[kb]); };
+  auto wait_tile = [&](bool newer_in_flight) { if (newer_in_flight) wait_all_but_two_tiles(); else wait_all(); };
+  if (wave < 4) {
+    for (int i = 0; i < n; ++i) {
+      const int cls = cls_of(i);
+      const bool work = active && !(cls & 2);  // nothing in a fully masked block is attended to
+      wait_tile(i + 1 < n);                    // K(i) landed (V(i), K(i+1) may still be in flight)
+      barrier();                               // barrier 4i
+      if (i >= 1 && i + 1 < n) issue_v(i + 1);
+      if (work) {
+        v16i acc[kKeyTiles];
+        v4i pk[kKeyTiles];
+        v16i oacc[kDSteps];
+        phase_gemm1(i, acc);
+        barrier();                             // barrier 4i+1
+        phase_softmax(i, cls, acc, pk);
+        wait_tile(i + 1 < n);                  // V(i) landed
+        barrier();                             // barrier 4i+2
+        if (i + 2 < n) issue_k(i + 2);
+        phase_gemm2(i, pk, oacc);
+        barrier();                             // barrier 4i+3
+        phase_merge(oacc);
+      } else {
+        barrier();
+        wait_tile(i + 1 < n);
+        barrier();
+        if (i + 2 < n) issue_k(i + 2);
+        barrier();
+      }
+    }
+    barrier();                                 // barrier 4n: wavefronts 4..7 run their last merge
+  } else {
+    wait_tile(n > 1);                          // K(0) landed
+    barrier();                                 // barrier 0
+    for (int i = 0; i < n; ++i) {
+      const int cls = cls_of(i);
+      const bool work = active && !(cls & 2);
+      barrier();                               // barrier 4i+1
+      if (work) {
+        v16i acc[kKeyTiles];
+        v4i pk[kKeyTiles];
+        v16i oacc[kDSteps];
+        phase_gemm1(i, acc);
+        wait_tile(i + 1 < n);                  // V(i) landed
+        barrier();                             // barrier 4i+2
+        if (i + 2 < n) issue_k(i + 2);
+        phase_softmax(i, cls, acc, pk);
+        barrier();                             // barrier 4i+3
+        phase_gemm2(i, pk, oacc);
+        wait_tile(i + 2 < n);                  // K(i+1) landed
+        barrier();                             // barrier 4(i+1)
+        if (i + 2 < n) issue_v(i + 2);
+        phase_merge(oacc);
+      } else {
+        wait_tile(i + 1 < n);
+        barrier();
+        if (i + 2 < n) issue_k(i + 2);
+        barrier();
+        wait_tile(i + 2 < n);
+        barrier();
+        if (i + 2 < n) issue_v(i + 2);
+      }
+    }
   }
+  if (!active) return;
 
   // ---- epilogue: normalise, requantise, store (inc/fmha_i8.cuh:318-332) --------------------------------------------
   // l_run sums 128 p / 32767 and O sums 128 p v, so mean(v) = O / (32767 l_run); a row with no unmasked key yields 0
   const float fin = (l_run > 0.f) ? args.out_scale * (128.f / kSnorm) / l_run : 0.f;
-  int8_t* op = args.o + head_off + (long)(qb * kBlockQ + wave * 32 + i32) * D + 4 * g;
+  int w[kDSteps][4];  // w[u][a]: the four int8 of output dims 32u + 8a + 4g .. +3 of query row i32
 #pragma unroll
   for (int u = 0; u < kDSteps; ++u)
 #pragma unroll
@@ -398,8 +502,24 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       // magic + y holds rne(y) in the low mantissa byte (round-half-even)
       const int lo = __builtin_amdgcn_perm(__float_as_int(y[1]), __float_as_int(y[0]), 0x0c0c0400);
       const int hi = __builtin_amdgcn_perm(__float_as_int(y[3]), __float_as_int(y[2]), 0x0c0c0400);
-      *reinterpret_cast<int*>(op + 32 * u + 8 * a) = __builtin_amdgcn_perm(hi, lo, 0x05040100);
+      w[u][a] = __builtin_amdgcn_perm(hi, lo, 0x05040100);
     }
+  // Lanes l and l+32 hold the g = 0 / g = 1 words of the same query row.  One v_permlane32_swap per word hands lane l
+  // both words of output tile u and lane l+32 both words of tile u+1: every lane then owns 32 contiguous bytes of a
+  // row and writes them with two 128-bit stores instead of eight scattered 32-bit ones.
+  int8_t* op = args.o + head_off + (long)(row0 + i32) * D + 32 * g;
+#pragma unroll
+  for (int u = 0; u < kDSteps; u += 2) {
+    int g0[4], g1[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const auto r = __builtin_amdgcn_permlane32_swap(w[u][a], w[u + 1][a], false, false);
+      g0[a] = r[0];
+      g1[a] = r[1];
+    }
+    *reinterpret_cast<v4i*>(op + 32 * u) = v4i{g0[0], g1[0], g0[1], g1[1]};
+    *reinterpret_cast<v4i*>(op + 32 * u + 16) = v4i{g0[2], g1[2], g0[3], g1[3]};
+  }
 }
 
 }  // namespace fmha_i8_gfx950
