@@ -57,14 +57,21 @@ int launch(hipStream_t stream, const FMHAParamI8& p, const AttnDataDescriptor& a
   // the price is that the exponent offset (1.5*2^23 + S)*c2 is then rounded on a coarser float grid.  Take that path
   // only while the offset stays below 2^12, i.e. while the rounding moves a whole row by less than 2^-13 in log2.
   const bool bias = (fmha_i8_gfx950::kMagic + 4194304.f) * fabsf(args.c2) < fmha_i8_gfx950::kBiasOffsetLimit;
+  // Folding the accumulator offset into the running O (see FASTACC in the kernel) costs a rounding of relative size
+  // 2^-24 at magnitude kMagic * sum(take) per key block; normalised by the row sum (>= sum(take)) and scaled to output
+  // LSBs that is at most about 0.0034 * (v_amax/o_amax) * sqrt(key blocks).  Take it while that stays below 0.1 LSB.
+  const float lsb_bound = 0.0034f * fabsf(p.v_amax / p.o_amax) * sqrtf((float)(a.seq_len / fmha_i8_gfx950::kBlockK));
+  const bool fast = lsb_bound < 0.1f;
   using namespace fmha_i8_gfx950;
+#define FMHA_LAUNCH(DD, BB, FF) hipLaunchKernelGGL((fmha_i8_fwd_kernel<DD, BB, FF>), grid, block, 0, stream, args)
   if (a.head_dim == 128) {
-    if (bias) hipLaunchKernelGGL((fmha_i8_fwd_kernel<128, true>), grid, block, 0, stream, args);
-    else hipLaunchKernelGGL((fmha_i8_fwd_kernel<128, false>), grid, block, 0, stream, args);
+    if (bias) { if (fast) FMHA_LAUNCH(128, true, true); else FMHA_LAUNCH(128, true, false); }
+    else { if (fast) FMHA_LAUNCH(128, false, true); else FMHA_LAUNCH(128, false, false); }
   } else {
-    if (bias) hipLaunchKernelGGL((fmha_i8_fwd_kernel<64, true>), grid, block, 0, stream, args);
-    else hipLaunchKernelGGL((fmha_i8_fwd_kernel<64, false>), grid, block, 0, stream, args);
+    if (bias) { if (fast) FMHA_LAUNCH(64, true, true); else FMHA_LAUNCH(64, true, false); }
+    else { if (fast) FMHA_LAUNCH(64, false, true); else FMHA_LAUNCH(64, false, false); }
   }
+#undef FMHA_LAUNCH
   const hipError_t err = hipGetLastError();
   return err == hipSuccess ? FMHA_I8_OK : FMHA_I8_ERR_HIP_BASE + (int)err;
 }

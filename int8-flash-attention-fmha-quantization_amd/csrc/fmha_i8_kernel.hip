@@ -99,7 +99,10 @@ __device__ __forceinline__ float half_sum(float x) {
 
 // BIAS: the S accumulators start at kMagicBits and are read as floats (no int->float convert).  Exact only while
 // (kMagic + |S|) * c2 stays small enough for the float grid; the host selects it from c2.
-template <int D, bool BIAS>
+// FASTACC: the running O absorbs the kMagic offset of the GEMM 2 accumulators (one fma per element and key block
+// instead of subtract + fma) and the offset is taken out once, in the epilogue.  O then lives near kMagic * sum(take)
+// and each merge rounds at that magnitude; the host enables it only where that rounding is far below one output LSB.
+template <int D, bool BIAS, bool FASTACC>
 __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelArgs args) {
   constexpr int kChunks = D / 16;                     // 16-byte chunks per row
   constexpr int kTileBytes = kBlockK * D;             // one K or V tile
@@ -231,6 +234,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #pragma unroll
     for (int r = 0; r < 16; ++r) o_f[u][r] = 0.f;
   float m_ref = args.floor2 - 2.f * kLazyLog2;  // reference exponent of the running O and l (base-2 units)
+  float t_run = 0.f;  // FASTACC: sum of the merge weights, i.e. how much of kMagic the running O carries
   float l_run = 0.f;                            // running row sum, in units of 1/128 (it sums 128*p)
   const float c2 = args.c2;
   const float bias_c2 = BIAS ? kMagic * c2 : 0.f;
@@ -400,6 +404,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       const float keep = __builtin_amdgcn_exp2f(m_ref - m_new);
       m_ref = m_new;
       l_run *= keep;
+      if (FASTACC) t_run *= keep;
 #pragma unroll
       for (int u = 0; u < kDSteps; ++u)
 #pragma unroll
@@ -407,12 +412,14 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     }
     const float take = __builtin_amdgcn_exp2f(m_blk - m_ref);
     l_run = __builtin_fmaf(take, l_blk, l_run);
+    if (FASTACC) t_run += take;
     const float neg_take = -take;  // P carries the sign: P = -128 p (inc/fmha_i8.cuh:298)
 #pragma unroll
     for (int u = 0; u < kDSteps; ++u)
 #pragma unroll
       for (int r = 0; r < 16; ++r)
-        o_f[u][r] = __builtin_fmaf(neg_take, __int_as_float(oacc[u][r]) - magic, o_f[u][r]);
+        o_f[u][r] = __builtin_fmaf(neg_take, FASTACC ? __int_as_float(oacc[u][r]) : __int_as_float(oacc[u][r]) - magic,
+                                   o_f[u][r]);
   };
 
   // ---- the tick schedule -------------------------------------------------------------------------------------------
@@ -491,6 +498,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // ---- epilogue: normalise, requantise, store (inc/fmha_i8.cuh:318-332) --------------------------------------------
   // l_run sums 128 p / 32767 and O sums 128 p v, so mean(v) = O / (32767 l_run); a row with no unmasked key yields 0
   const float fin = (l_run > 0.f) ? args.out_scale * (128.f / kSnorm) / l_run : 0.f;
+  const float corr = FASTACC ? magic * t_run : 0.f;
   int w[kDSteps][4];  // w[u][a]: the four int8 of output dims 32u + 8a + 4g .. +3 of query row i32
 #pragma unroll
   for (int u = 0; u < kDSteps; ++u)
@@ -498,7 +506,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     for (int a = 0; a < 4; ++a) {
       float y[4];
 #pragma unroll
-      for (int bb = 0; bb < 4; ++bb) y[bb] = __builtin_amdgcn_fmed3f(o_f[u][4 * a + bb] * fin, -127.f, 127.f) + magic;
+      for (int bb = 0; bb < 4; ++bb) y[bb] = __builtin_amdgcn_fmed3f((o_f[u][4 * a + bb] + corr) * fin, -127.f, 127.f) + magic;
       // magic + y holds rne(y) in the low mantissa byte (round-half-even)
       const int lo = __builtin_amdgcn_perm(__float_as_int(y[1]), __float_as_int(y[0]), 0x0c0c0400);
       const int hi = __builtin_amdgcn_perm(__float_as_int(y[3]), __float_as_int(y[2]), 0x0c0c0400);
