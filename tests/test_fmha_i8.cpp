@@ -9,6 +9,8 @@
 //                                           uniform(+-0.5) Q/K, |uniform| V, scattered 20 % mask, o_amax measured
 //   test_fmha_i8 --B 2 --H 4 --S 512 --d 64 [--valid L] [--dist normal|student_t|reference]
 //   common: --seed N --iters N --cpu-heads N (0 = all) --cpu-threads N --json FILE --no-check
+//   --calibrate-copy MiB   also run one device-to-device copy of that size, so that a counter run (FETCH_SIZE /
+//                          WRITE_SIZE) sees a plain copy kernel of known traffic to scale the attention kernel's by
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
@@ -264,6 +266,7 @@ int main(int argc, char** argv) {
   std::vector<Case> cases;
   Case custom;
   bool have_custom = false;
+  long calib_mib = 0;
   for (int i = 1; i < argc; ++i) {
     const std::string a = argv[i];
     auto val = [&]() -> const char* {
@@ -295,6 +298,7 @@ int main(int argc, char** argv) {
     else if (a == "--cpu-threads") opt.cpu_threads = atoi(val());
     else if (a == "--no-check") opt.check = false;
     else if (a == "--json") opt.json = val();
+    else if (a == "--calibrate-copy") calib_mib = atol(val());
     else {
       fprintf(stderr, "unknown argument %s\n", a.c_str());
       return 2;
@@ -311,6 +315,17 @@ int main(int argc, char** argv) {
   printf("%s | device %s, %d CUs, %.0f MHz -> CU*8192*clk = %.1f int8 TOPS | host threads %u\n", FMHAInferI8Version(),
          prop.gcnArchName, prop.multiProcessorCount, prop.clockRate / 1e3,
          prop.multiProcessorCount * 8192.0 * prop.clockRate * 1e3 / 1e12, std::thread::hardware_concurrency());
+  if (calib_mib > 0) {
+    void *src, *dst;
+    const size_t bytes = (size_t)calib_mib << 20;
+    CHECK_HIP(hipMalloc(&src, bytes)), CHECK_HIP(hipMalloc(&dst, bytes));
+    CHECK_HIP(hipMemset(src, 1, bytes));
+    CHECK_HIP(hipDeviceSynchronize());
+    CHECK_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToDevice));
+    CHECK_HIP(hipDeviceSynchronize());
+    CHECK_HIP(hipFree(src)), CHECK_HIP(hipFree(dst));
+    printf("calibration copy: %ld MiB device to device (reads %zu bytes, writes %zu bytes)\n", calib_mib, bytes, bytes);
+  }
   FILE* json = opt.json.empty() ? nullptr : fopen(opt.json.c_str(), "w");
   bool all = true;
   for (const Case& c : cases) all = run_case(c, opt, json) && all;
