@@ -53,12 +53,13 @@ int launch(hipStream_t stream, const FMHAParamI8& p, const AttnDataDescriptor& a
   args.masked2 = -1000000.f * args.c2;
   args.out_scale = p.v_amax / (p.o_amax * 128.f);  // inc/fmha_i8.cuh:318
   const dim3 grid((unsigned)args.total_wgs), block(fmha_i8_gfx950::kThreads);
-  // The accumulators of Q.K^T can be read as floats without a convert when they start at the bit pattern of 1.5*2^23;
-  // the price is that the exponent offset (1.5*2^23 + S)*c2 is then rounded on a coarser float grid.  Take that path
+  // The accumulators of Q.K^T can be read as floats without a convert when they start at the bit pattern of kBase;
+  // the price is that the exponent offset (kBase*2^26 + S)*c2 is then rounded on a coarser float grid.  Take that path
   // only while the offset stays below 2^12, i.e. while the rounding moves a whole row by less than 2^-13 in log2.
-  const bool bias = (fmha_i8_gfx950::kMagic + 4194304.f) * fabsf(args.c2) < fmha_i8_gfx950::kBiasOffsetLimit;
+  const bool bias = (fmha_i8_gfx950::kBase * fmha_i8_gfx950::kBaseScale + 4194304.f) * fabsf(args.c2) <
+                    fmha_i8_gfx950::kBiasOffsetLimit;
   // Folding the accumulator offset into the running O (see FASTACC in the kernel) costs a rounding of relative size
-  // 2^-24 at magnitude kMagic * sum(take) per key block; normalised by the row sum (>= sum(take)) and scaled to output
+  // 2^-24 at magnitude kBase * sum(take) per key block; normalised by the row sum (>= sum(take)) and scaled to output
   // LSBs that is at most about 0.0034 * (v_amax/o_amax) * sqrt(key blocks).  Take it while that stays below 0.1 LSB.
   const float lsb_bound = 0.0034f * fabsf(p.v_amax / p.o_amax) * sqrtf((float)(a.seq_len / fmha_i8_gfx950::kBlockK));
   const bool fast = lsb_bound < 0.1f;

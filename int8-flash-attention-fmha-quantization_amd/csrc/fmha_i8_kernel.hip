@@ -22,8 +22,8 @@
 //     wavefronts 0..3, so an MFMA phase of one always overlaps a VALU phase of the other on the same SIMD;
 //   * the softmax is written for instruction count: exp in the base-2 domain with every scale folded into one fma,
 //     v_max3 on the raw accumulators for the row maximum, P converted two at a time by v_cvt_pknorm_i16_f32 and packed
-//     by v_perm_b32, the int32 accumulators of both GEMMs start at the bit pattern of 1.5*2^23 so that they can be
-//     read as floats without a convert, the running O is only rescaled when a row maximum jumps by more than
+//     by v_perm_b32, the int32 accumulators of both GEMMs start at the bit pattern of a float (an MFMA inline constant)
+//     so that they can be read as floats without a convert, the running O is only rescaled when a row maximum jumps by more than
 //     2^kLazyLog2, and O is normalised once, in the epilogue.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -39,8 +39,14 @@ constexpr int kBlockK = 128;   // keys per softmax block (the reference's BASE_S
 constexpr int kThreads = 512;  // 8 wavefronts: 0..3 and 4..7 run the key-block phases one phase apart
 constexpr int kXcds = 8;
 constexpr int kMaxKeyBlocks = 512;       // seq_len <= 65536
-constexpr float kMagic = 12582912.0f;    // 1.5 * 2^23: float whose low mantissa bits hold a small signed integer
-constexpr int kMagicBits = 0x4B400000;   // its bit pattern; kMagicBits + n is the float kMagic + n for |n| < 2^22
+constexpr float kMagic = 12582912.0f;    // 1.5 * 2^23: kMagic + y holds rne(y) in its low mantissa bits (output rounding)
+// Both GEMMs start their int32 accumulators at the bit pattern of the float 1/(2 pi), which the MFMA takes as an INLINE
+// CONSTANT C operand (no registers, no moves).  That float sits 2292099 ulps above 2^-3 and 6096509 below 2^-2, more than
+// any int8 dot product of 128 terms can reach (|x| <= 2^21), so kBaseBits + x read as a float is exactly
+// kBase + x * 2^-26: the integer result is available to float arithmetic without a convert.
+constexpr int kBaseBits = 0x3E22F983;
+constexpr float kBase = __builtin_bit_cast(float, kBaseBits);
+constexpr float kBaseScale = 67108864.0f;  // 2^26: float units per integer unit, inverted
 constexpr float kBiasOffsetLimit = 4096.0f;  // see the launch code: bound on the exponent offset of the biased path
 constexpr float kLog2Pscale = -7.99995597f;  // log2(128 / 32767): exp2(x + kLog2Pscale) = 128 p / 32767
 constexpr float kLazyLog2 = 10.0f;       // the running O is rescaled only when a row maximum grows by more than this
@@ -97,10 +103,10 @@ __device__ __forceinline__ float half_sum(float x) {
   return __int_as_float(r[0]) + __int_as_float(r[1]);
 }
 
-// BIAS: the S accumulators start at kMagicBits and are read as floats (no int->float convert).  Exact only while
-// (kMagic + |S|) * c2 stays small enough for the float grid; the host selects it from c2.
-// FASTACC: the running O absorbs the kMagic offset of the GEMM 2 accumulators (one fma per element and key block
-// instead of subtract + fma) and the offset is taken out once, in the epilogue.  O then lives near kMagic * sum(take)
+// BIAS: the S accumulators start at kBaseBits and are read as floats (no int->float convert).  Exact only while
+// (kBase * 2^26 + |S|) * c2 stays small enough for the float grid; the host selects it from c2.
+// FASTACC: the running O absorbs the kBase offset of the GEMM 2 accumulators (one fma per element and key block
+// instead of subtract + fma) and the offset is taken out once, in the epilogue.  O then lives near kBase * sum(take)
 // and each merge rounds at that magnitude; the host enables it only where that rounding is far below one output LSB.
 template <int D, bool BIAS, bool FASTACC>
 __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelArgs args) {
@@ -138,8 +144,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   const int8_t* __restrict__ mg = args.mask + (long)b * S;
   const int n_blocks = S / kBlockK;
 
-  // The prologue puts every cold miss in flight before it waits for any of them: the first two K/V tiles (tile 1 on
-  // speculation: it exists whenever seq_len >= 256, whether or not its keys are masked), the Q rows, and the mask bytes.
+  // The prologue puts every cold miss in flight before it waits for any of them: the mask bytes, the first two K/V
+  // tiles (tile 1 on speculation: it exists whenever seq_len >= 256, whether or not its keys are masked) and the Q rows.
   // ---- per-lane addressing -----------------------------------------------------------------------------------------
   // direct-to-LDS loads: lane l of a 1 KiB region lands at byte 16*l of the region, so the lane FETCHES the chunk that
   // the swizzle assigns to that slot.
@@ -191,27 +197,41 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   auto wait_all = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
   auto barrier = [&]() { asm volatile("s_barrier" ::: "memory"); };
 
-  issue_k(0);
-  issue_v(0);
-  if (n_blocks > 1) { issue_k(1); issue_v(1); }
-
-  // ---- Q: B operand of GEMM 1, loaded once -----------------------------------------------------------------------
+  // Loads of the prologue, all issued before any is waited for and all by inline assembly, so that every wait is an
+  // explicit s_waitcnt vmcnt(n) that counts the loads still allowed in flight (memory reads return in issue order):
+  //   mask bytes of the first 2048 keys (1 load) | K0 | Q (kDSteps loads) | V0
+  // (K1 and V1 follow right after the first barrier: the CU's vector memory path moves 64 bytes per cycle, and
+  // everything queued here delays the first GEMM.)
   const int row0 = qb * kBlockQ + wave * 32;  // first query row of this wavefront
   const bool active = row0 < S;               // seq_len is a multiple of 128, not of 256: the last workgroup may be half empty
-  v4i qreg[kDSteps];
-#pragma unroll
-  for (int kk = 0; kk < kDSteps; ++kk) qreg[kk] = v4i{0, 0, 0, 0};
-  if (active) {
-    const int8_t* qp = args.q + head_off + (long)(row0 + i32) * D + 16 * g;
-#pragma unroll
-    for (int kk = 0; kk < kDSteps; ++kk) qreg[kk] = *reinterpret_cast<const v4i*>(qp + 32 * kk);
+  int mask_word;
+  {
+    const int j = 4 * tid < S ? 4 * tid : S - 4;
+    asm volatile("global_load_dword %0, %1, %2" : "=v"(mask_word) : "v"(j), "s"(mg) : "memory");
   }
+  issue_k(0);
+  v4i qreg[kDSteps];  // Q: B operand of GEMM 1, loaded once
+  {
+    // wavefronts past the end of the sequence load row 0 (unused) so that every wavefront has the same loads in flight
+    const int8_t* qp = args.q + head_off;
+    const int qoff = ((active ? row0 : 0) + i32) * D + 16 * g;
+#pragma unroll
+    for (int kk = 0; kk < kDSteps; ++kk)
+      asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(qreg[kk]) : "v"(qoff + 32 * kk), "s"(qp) : "memory");
+  }
+  issue_v(0);
 
   // ---- classify the key blocks of this batch entry: 4 mask bytes per lane, two blocks per wavefront ballot ---------
+  asm volatile("s_waitcnt vmcnt(%1)" : "+v"(mask_word) : "n"(2 * kRegionsPerWave + kDSteps) : "memory");
   for (int base = 0; base < S; base += 4 * kThreads) {
     const int j = base + 4 * tid;
     int nib = 15;
-    if (j < S) nib = (mg[j] != 0 ? 1 : 0) | (mg[j + 1] != 0 ? 2 : 0) | (mg[j + 2] != 0 ? 4 : 0) | (mg[j + 3] != 0 ? 8 : 0);
+    if (base == 0) {
+      const unsigned w = (unsigned)mask_word;
+      if (j < S) nib = ((w & 0xffu) ? 1 : 0) | ((w & 0xff00u) ? 2 : 0) | ((w & 0xff0000u) ? 4 : 0) | ((w & 0xff000000u) ? 8 : 0);
+    } else if (j < S) {
+      nib = (mg[j] != 0 ? 1 : 0) | (mg[j + 1] != 0 ? 2 : 0) | (mg[j + 2] != 0 ? 4 : 0) | (mg[j + 3] != 0 ? 8 : 0);
+    }
     const unsigned long long some = __ballot(nib != 0), all = __ballot(nib == 15);
     if ((lane & 31) == 0 && j < S) {
       const unsigned half_some = (unsigned)(some >> (lane & 32)), half_all = (unsigned)(all >> (lane & 32));
@@ -234,98 +254,140 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #pragma unroll
     for (int r = 0; r < 16; ++r) o_f[u][r] = 0.f;
   float m_ref = args.floor2 - 2.f * kLazyLog2;  // reference exponent of the running O and l (base-2 units)
-  float t_run = 0.f;  // FASTACC: sum of the merge weights, i.e. how much of kMagic the running O carries
+  float t_run = 0.f;  // FASTACC: sum of the merge weights, i.e. how much of kBase the running O carries
   float l_run = 0.f;                            // running row sum, in units of 1/128 (it sums 128*p)
-  const float c2 = args.c2;
-  const float bias_c2 = BIAS ? kMagic * c2 : 0.f;
+  const float c2 = BIAS ? args.c2 * kBaseScale : args.c2;  // exponent per unit of sf() below
+  const float bias_c2 = BIAS ? kBase * c2 : 0.f;
   float magic = kMagic;
   asm volatile("" : "+v"(magic));  // a register operand: as a literal it would double the size of every instruction using it
-  v16i magic_c;  // C operand that starts an accumulation chain at kMagicBits without per-element moves
-#pragma unroll
-  for (int r = 0; r < 16; ++r) magic_c[r] = kMagicBits;
-  asm volatile("" : "+v"(magic_c));  // keep it in registers: 16 moves once, not 128 per key block
+  const v16i base_c = {kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits,
+                       kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits};
 
-  // Make the compiler retire its own outstanding loads (Q) here: its later vmcnt bookkeeping does not know about the
-  // hand-issued LDS-DMA loads and would otherwise wait for them inside the loop.
+  // K0 and Q have landed once at most V0 is still in flight.  The registers are redefined after the wait so that no
+  // use of them can be scheduled above it.
+  asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kRegionsPerWave) : "memory");
 #pragma unroll
-  for (int kk = 0; kk < kDSteps; ++kk) asm volatile("" ::"v"(qreg[kk]));
+  for (int kk = 0; kk < kDSteps; ++kk) asm volatile("" : "+v"(qreg[kk]));
 
   // ---- the four phases of one key block ----------------------------------------------------------------------------
   // acc:  S^T, for query column i32 keys 32t + 8a + 4g + bb at acc[t][4a+bb]        (GEMM 1 -> softmax)
   // pk:   P^T, int8, B operand of GEMM 2                                              (softmax -> GEMM 2)
-  // oacc: O~^T, output dims 32u + 8a + 4g + bb at oacc[u][4a+bb], as kMagic + O~      (GEMM 2 -> merge)
+  // oacc: O~^T, output dims 32u + 8a + 4g + bb at oacc[u][4a+bb], as kBaseBits + O~   (GEMM 2 -> merge)
   float m_blk = 0.f;    // block-local row maximum, base-2 units
   float l_blk = 0.f;    // sum of (128/32767) p over this lane's keys
 
-  // GEMM 1: S^T[key][query] = K . Q^T, int32 (inc/fmha_i8.cuh:120-172)
-  auto phase_gemm1 = [&](int kb, v16i (&acc)[kKeyTiles]) {
+  // Row maximum of one finished 32-key tile, folded into two independent chains (integer compare: monotone in the
+  // score, also for the biased bit patterns).
+  auto tile_max = [&](const v16i& a, int (&mx)[2], bool first) {
+    if (first) {
+      mx[0] = max(max(a[0], a[1]), a[2]);
+      mx[1] = max(max(a[8], a[9]), a[10]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        mx[0] = max(max(mx[0], a[3 + 2 * j]), a[4 + 2 * j]);
+        mx[1] = max(max(mx[1], a[11 + 2 * j]), a[12 + 2 * j]);
+      }
+      mx[0] = max(mx[0], a[7]);
+      mx[1] = max(mx[1], a[15]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        mx[0] = max(max(mx[0], a[2 * j]), a[2 * j + 1]);
+        mx[1] = max(max(mx[1], a[8 + 2 * j]), a[9 + 2 * j]);
+      }
+    }
+  };
+
+  // GEMM 1: S^T[key][query] = K . Q^T, int32 (inc/fmha_i8.cuh:120-172), one 32-key tile after the other; the row
+  // maximum of tile t-1 is taken while the MFMAs of tile t run.  mx covers tiles 0 .. kKeyTiles-2 on return.
+  auto phase_gemm1 = [&](int kb, v16i (&acc)[kKeyTiles], int (&mx)[2]) {
     const int8_t* lds_k = &lds[kb & 1][0][0];
     const v16i zero_c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    v4i ka[2][kKeyTiles];  // operand reads run one k-step ahead of the MFMAs that consume them
+    v4i ka[2][kDSteps];  // operand reads run one key tile ahead of the MFMAs that consume them
 #pragma unroll
-    for (int t = 0; t < kKeyTiles; ++t) ka[0][t] = *reinterpret_cast<const v4i*>(lds_k + k_read_off[0] + 32 * t * D);
+    for (int kk = 0; kk < kDSteps; ++kk) ka[0][kk] = *reinterpret_cast<const v4i*>(lds_k + k_read_off[kk]);
 #pragma unroll
-    for (int kk = 0; kk < kDSteps; ++kk) {
-      if (kk + 1 < kDSteps) {
+    for (int t = 0; t < kKeyTiles; ++t) {
+      if (t + 1 < kKeyTiles) {
 #pragma unroll
-        for (int t = 0; t < kKeyTiles; ++t)
-          ka[(kk + 1) & 1][t] = *reinterpret_cast<const v4i*>(lds_k + k_read_off[kk + 1] + 32 * t * D);
+        for (int kk = 0; kk < kDSteps; ++kk)
+          ka[(t + 1) & 1][kk] = *reinterpret_cast<const v4i*>(lds_k + k_read_off[kk] + 32 * (t + 1) * D);
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int t = 0; t < kKeyTiles; ++t)
-        acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ka[kk & 1][t], qreg[kk],
-                                                       kk == 0 ? (BIAS ? magic_c : zero_c) : acc[t], 0, 0, 0);
+      for (int kk = 0; kk < kDSteps; ++kk)
+        acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ka[t & 1][kk], qreg[kk],
+                                                       kk == 0 ? (BIAS ? base_c : zero_c) : acc[t], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
+      if (t >= 1) {
+        tile_max(acc[t - 1], mx, t == 1);
+        asm volatile("" : "+v"(mx[0]), "+v"(mx[1]));  // keeps these few instructions here, in the shadow of the MFMAs
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   };
-  // (sf(t,r) below: the score as a float; with BIAS it still carries +kMagic, which the exponent offset removes.)
+  // (sf(t,r) below: the score as a float; with BIAS that is kBase + S * 2^-26, and the exponent offset removes kBase.)
   // block softmax (inc/fmha_i8.cuh:174-253)
-  auto phase_softmax = [&](int kb, int cls, const v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles]) {
+  auto phase_softmax = [&](int kb, int cls, const v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles], int (&mx)[2]) {
     auto sf = [&](int t, int r) -> float { return BIAS ? __int_as_float(acc[t][r]) : (float)acc[t][r]; };
     l_blk = 0.f;
     if (cls == 0) {
-      // integer maximum (monotone in the score, also for the biased bit patterns), two independent chains
-      constexpr int kVals = 16 * kKeyTiles;  // scores per lane; v(n) = acc[n / 16][n % 16]
-      int t0 = acc[0][0], t1 = acc[0][1];
-#pragma unroll
-      for (int n = 2; n + 3 < kVals; n += 4) {
-        t0 = max(max(t0, acc[n / 16][n % 16]), acc[(n + 1) / 16][(n + 1) % 16]);
-        t1 = max(max(t1, acc[(n + 2) / 16][(n + 2) % 16]), acc[(n + 3) / 16][(n + 3) % 16]);
-      }
-      t0 = max(max(t0, acc[kKeyTiles - 1][14]), acc[kKeyTiles - 1][15]);
-      const int ti = half_max(max(t0, t1));
+      tile_max(acc[kKeyTiles - 1], mx, false);
+      const int ti = half_max(max(mx[0], mx[1]));
       const float top = BIAS ? __int_as_float(ti) : (float)ti;
       // off = top*c2 rounded; p' = exp2(s*c2 - off) = p * 2^(resid) with one row-wide resid below 1 ulp of off, and the
-      // block maximum that is consistent with p' is off itself (minus the constant kMagic*c2 when BIAS).
+      // block maximum that is consistent with p' is off itself (minus the constant kBase*c2 when BIAS).
       float off = top * c2;
       if (!BIAS) off = fmaxf(off, args.floor2);
       m_blk = off - bias_c2;
       const float offq = off - kLog2Pscale;  // exp2(x - offq) = 128 p / 32767: the snorm conversion returns rne(128 p)
-      // Three stages per 32-key tile - 16 fma, 16 exp, then sums and packing - software-pipelined one tile apart and
-      // fenced for the scheduler, so that every instruction is far from the one whose result it needs: a wavefront
-      // issues in order and a transcendental takes several issue slots to deliver.
-      float e[2][16];
-      auto stage_exp = [&](int t) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) e[t & 1][r] = __builtin_fmaf(sf(t, r), c2, -offq);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) e[t & 1][r] = __builtin_amdgcn_exp2f(e[t & 1][r]);
-        __builtin_amdgcn_sched_barrier(0);
+      // Software pipeline over quads of four scores (quad qd = 4 t + a): step s issues the four exponentials of quad s
+      // with the four scaling fmas of quad s+1 and the sums and packing of quad s-1 between them.  A wavefront issues in
+      // order, a transcendental occupies its unit for about two issue slots, and an instruction that follows one without
+      // needing the unit goes out in its shadow; the fences make the scheduler keep this order.
+      constexpr int kQuads = 4 * kKeyTiles;
+      float x[3][4];  // x[qd % 3]: scaled exponents, then exponentials, of quad qd
+      auto q_fma = [&](int qd, int j) {
+        x[qd % 3][j] = __builtin_fmaf(sf(qd / 4, 4 * (qd % 4) + j), c2, -offq);
       };
-      stage_exp(0);
+      auto q_exp = [&](int qd, int j) { x[qd % 3][j] = __builtin_amdgcn_exp2f(x[qd % 3][j]); };
+      float s01 = 0.f, s23 = 0.f;
+      v2s lo, hi;
+      auto q_out = [&](int qd, int j) {  // seven steps of sums and packing of quad qd
+        const float(&e)[4] = x[qd % 3];
+        if (j == 0) s01 = e[0] + e[1];
+        if (j == 1) s23 = e[2] + e[3];
+        if (j == 2) lo = __builtin_amdgcn_cvt_pknorm_i16(-e[0], -e[1]);
+        if (j == 3) hi = __builtin_amdgcn_cvt_pknorm_i16(-e[2], -e[3]);
+        if (j == 4) s01 += s23;
+        if (j == 5) pk[qd / 4][qd % 4] = __builtin_amdgcn_perm(__builtin_bit_cast(int, hi), __builtin_bit_cast(int, lo), 0x06040200);
+        if (j == 6) l_blk += s01;
+      };
+      if (kQuads > 0) {
 #pragma unroll
-      for (int t = 0; t < kKeyTiles; ++t) {
-        if (t + 1 < kKeyTiles) stage_exp(t + 1);
-        const float(&et)[16] = e[t & 1];
-#pragma unroll
-        for (int a = 0; a < 4; ++a) {
-          l_blk += (et[4 * a] + et[4 * a + 1]) + (et[4 * a + 2] + et[4 * a + 3]);
-          pk[t][a] = pack4_snorm(-et[4 * a], -et[4 * a + 1], -et[4 * a + 2], -et[4 * a + 3]);
-        }
+        for (int j = 0; j < 4; ++j) q_fma(0, j);
         __builtin_amdgcn_sched_barrier(0);
       }
+#pragma unroll
+      for (int s = 0; s <= kQuads; ++s) {
+        const bool ex = s < kQuads, fm = s + 1 < kQuads, out = s >= 1;
+        auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
+        if (ex) { q_exp(s, 0); fence(); }
+        if (fm) { q_fma(s + 1, 0); q_fma(s + 1, 1); }
+        if (out) q_out(s - 1, 0);
+        fence();
+        if (ex) { q_exp(s, 1); fence(); }
+        if (fm) { q_fma(s + 1, 2); q_fma(s + 1, 3); }
+        if (out) q_out(s - 1, 1);
+        fence();
+        if (ex) { q_exp(s, 2); fence(); }
+        if (out) { q_out(s - 1, 2); q_out(s - 1, 3); q_out(s - 1, 4); }
+        fence();
+        if (ex) { q_exp(s, 3); fence(); }
+        if (out) { q_out(s - 1, 5); q_out(s - 1, 6); }
+        fence();
+      }
+      l_blk = half_sum(l_blk);
     } else {
       // some keys of this block are masked out (nonzero mask byte, inc/fmha_i8.cuh:189-192,216-221)
       const int8_t* mp = mg + kb * kBlockK + 4 * i32;
@@ -361,11 +423,11 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
           }
           pk[t][a] = pack4_snorm(-e[0], -e[1], -e[2], -e[3]);
         }
+      l_blk = half_sum(l_blk);
     }
-    l_blk = half_sum(l_blk);
   };
 
-  // GEMM 2: O~^T[d][query] = V^T . P^T, int32 (inc/fmha_i8.cuh:255-296); accumulators start at kMagicBits
+  // GEMM 2: O~^T[d][query] = V^T . P^T, int32 (inc/fmha_i8.cuh:255-296); accumulators start at kBaseBits
   auto phase_gemm2 = [&](int kb, const v4i (&pk)[kKeyTiles], v16i (&oacc)[kDSteps]) {
     const int8_t* lds_v = &lds[kb & 1][1][0];
     typedef v2i __attribute__((address_space(3))) * lds_v2i_ptr;
@@ -390,7 +452,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #pragma unroll
       for (int u = 0; u < kDSteps; ++u) {
         const v4i a = {va[t & 1][u][0][0], va[t & 1][u][0][1], va[t & 1][u][1][0], va[t & 1][u][1][1]};
-        oacc[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, pk[t], t == 0 ? magic_c : oacc[u], 0, 0, 0);
+        oacc[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, pk[t], t == 0 ? base_c : oacc[u], 0, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -413,12 +475,13 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     const float take = __builtin_amdgcn_exp2f(m_blk - m_ref);
     l_run = __builtin_fmaf(take, l_blk, l_run);
     if (FASTACC) t_run += take;
-    const float neg_take = -take;  // P carries the sign: P = -128 p (inc/fmha_i8.cuh:298)
+    float neg_take = -take;  // P carries the sign: P = -128 p (inc/fmha_i8.cuh:298)
+    asm volatile("" : "+v"(neg_take));  // a plain register operand: as a source modifier it would force the 64-bit encoding
 #pragma unroll
     for (int u = 0; u < kDSteps; ++u)
 #pragma unroll
       for (int r = 0; r < 16; ++r)
-        o_f[u][r] = __builtin_fmaf(neg_take, FASTACC ? __int_as_float(oacc[u][r]) : __int_as_float(oacc[u][r]) - magic,
+        o_f[u][r] = __builtin_fmaf(neg_take, FASTACC ? __int_as_float(oacc[u][r]) : __int_as_float(oacc[u][r]) - kBase,
                                    o_f[u][r]);
   };
 
@@ -435,16 +498,20 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     for (int i = 0; i < n; ++i) {
       const int cls = cls_of(i);
       const bool work = active && !(cls & 2);  // nothing in a fully masked block is attended to
-      wait_tile(i + 1 < n);                    // K(i) landed (V(i), K(i+1) may still be in flight)
+      if (i > 0) wait_tile(i + 1 < n);         // K(i) landed (V(i), K(i+1) may still be in flight); K(0): prologue
       barrier();                               // barrier 4i
-      if (i >= 1 && i + 1 < n) issue_v(i + 1);
+      if (i + 1 < n) {
+        if (i == 0) issue_k(1);
+        issue_v(i + 1);
+      }
       if (work) {
         v16i acc[kKeyTiles];
         v4i pk[kKeyTiles];
         v16i oacc[kDSteps];
-        phase_gemm1(i, acc);
+        int mx[2];
+        phase_gemm1(i, acc, mx);
         barrier();                             // barrier 4i+1
-        phase_softmax(i, cls, acc, pk);
+        phase_softmax(i, cls, acc, pk, mx);
         wait_tile(i + 1 < n);                  // V(i) landed
         barrier();                             // barrier 4i+2
         if (i + 2 < n) issue_k(i + 2);
@@ -461,8 +528,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     }
     barrier();                                 // barrier 4n: wavefronts 4..7 run their last merge
   } else {
-    wait_tile(n > 1);                          // K(0) landed
-    barrier();                                 // barrier 0
+    barrier();                                 // barrier 0 (K(0) landed: prologue)
+    if (n > 1) { issue_k(1); issue_v(1); }
     for (int i = 0; i < n; ++i) {
       const int cls = cls_of(i);
       const bool work = active && !(cls & 2);
@@ -471,11 +538,12 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         v16i acc[kKeyTiles];
         v4i pk[kKeyTiles];
         v16i oacc[kDSteps];
-        phase_gemm1(i, acc);
+        int mx[2];
+        phase_gemm1(i, acc, mx);
         wait_tile(i + 1 < n);                  // V(i) landed
         barrier();                             // barrier 4i+2
         if (i + 2 < n) issue_k(i + 2);
-        phase_softmax(i, cls, acc, pk);
+        phase_softmax(i, cls, acc, pk, mx);
         barrier();                             // barrier 4i+3
         phase_gemm2(i, pk, oacc);
         wait_tile(i + 2 < n);                  // K(i+1) landed
@@ -493,12 +561,13 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       }
     }
   }
+  wait_all();  // nothing may still be writing LDS when the wavefront ends (only possible when every key is masked)
   if (!active) return;
 
   // ---- epilogue: normalise, requantise, store (inc/fmha_i8.cuh:318-332) --------------------------------------------
   // l_run sums 128 p / 32767 and O sums 128 p v, so mean(v) = O / (32767 l_run); a row with no unmasked key yields 0
-  const float fin = (l_run > 0.f) ? args.out_scale * (128.f / kSnorm) / l_run : 0.f;
-  const float corr = FASTACC ? magic * t_run : 0.f;
+  const float fin = (l_run > 0.f) ? args.out_scale * (128.f / kSnorm) * kBaseScale / l_run : 0.f;
+  const float corr = FASTACC ? kBase * t_run : 0.f;
   int w[kDSteps][4];  // w[u][a]: the four int8 of output dims 32u + 8a + 4g .. +3 of query row i32
 #pragma unroll
   for (int u = 0; u < kDSteps; ++u)

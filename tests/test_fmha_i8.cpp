@@ -8,7 +8,7 @@
 //   test_fmha_i8 --sweep                    the reference's own sweep: B=H=1, S in {128..4096 step per its list}, d in {64,128},
 //                                           uniform(+-0.5) Q/K, |uniform| V, scattered 20 % mask, o_amax measured
 //   test_fmha_i8 --B 2 --H 4 --S 512 --d 64 [--valid L] [--dist normal|student_t|reference]
-//   common: --seed N --iters N --cpu-heads N (0 = all) --cpu-threads N --json FILE --no-check
+//   common: --seed N --iters N --warmup N --cpu-heads N (0 = all) --cpu-threads N --json FILE --no-check
 //   --calibrate-copy MiB   also run one device-to-device copy of that size, so that a counter run (FETCH_SIZE /
 //                          WRITE_SIZE) sees a plain copy kernel of known traffic to scale the attention kernel's by
 #include <hip/hip_runtime_api.h>
@@ -83,7 +83,8 @@ Case config_case(int id) {
 
 struct Options {
   uint64_t seed = 2023;  // test_fmha_i8.cpp:49
-  int iters = 200;
+  int iters = 1000;
+  int warmup = 1500;
   long cpu_heads = 8;
   int cpu_threads = 0;
   bool check = true;
@@ -182,7 +183,8 @@ bool run_case(const Case& c, const Options& opt, FILE* json) {
     fprintf(stderr, "launch failed: %s\n", FMHAInferI8StatusString(st));
     return false;
   }
-  for (int i = 0; i < 3; ++i) gpuImpl::FMHAInferI8(stream, param, desc, dq, dk, dv, dm, dout, true);
+  // warm-up: the shader clock needs tens of milliseconds of load to settle (a cold call is up to 30 % slower)
+  for (int i = 0; i < opt.warmup; ++i) gpuImpl::FMHAInferI8(stream, param, desc, dq, dk, dv, dm, dout, true);
   CHECK_HIP(hipStreamSynchronize(stream));
   hipEvent_t e0, e1;
   CHECK_HIP(hipEventCreate(&e0)), CHECK_HIP(hipEventCreate(&e1));
@@ -294,6 +296,7 @@ int main(int argc, char** argv) {
     else if (a == "--dist") custom.dist = val();
     else if (a == "--seed") opt.seed = strtoull(val(), nullptr, 10);
     else if (a == "--iters") opt.iters = atoi(val());
+    else if (a == "--warmup") opt.warmup = atoi(val());
     else if (a == "--cpu-heads") opt.cpu_heads = atol(val());
     else if (a == "--cpu-threads") opt.cpu_threads = atoi(val());
     else if (a == "--no-check") opt.check = false;
