@@ -115,6 +115,6 @@ const char* FMHAInferI8StatusString(int status) {
   return "unknown status";
 }
 
-const char* FMHAInferI8Version(void) { return "fmha_i8 gfx950 mfma32x32x32 direct-to-lds anti-phase"; }
+const char* FMHAInferI8Version(void) { return "fmha_i8 gfx950 mfma32x32x32 direct-to-lds two-phase"; }
 
 }  // extern "C"

@@ -11,20 +11,23 @@
 //   * both GEMMs run on v_mfma_i32_32x32x32_i8 in the TRANSPOSED formulation S^T = K.Q^T and O^T = V^T.P^T: each
 //     lane then owns one query column, so the row max / row sum are in-register reductions plus one exchange with
 //     lane^32, and the quantised P^T tile leaves the accumulator already in the B-operand register layout;
-//   * K and V tiles of 128 keys go HBM -> LDS directly (global_load_lds_dwordx4, no VGPR staging, no ds_write),
-//     double buffered and fetched two key blocks ahead, as [key][d] with the 16-byte chunk index XOR-swizzled by the
-//     row (the swizzle is applied to the global address each lane fetches), so that the 128-bit operand reads of K and
-//     the transposing reads of V (ds_read_b64_tr_b8) are bank-conflict free; Q goes once per workgroup straight into
-//     MFMA operand registers;
-//   * the kernel is bound by the VALU issue port (a wavefront issues one VALU instruction per ~4.5 cycles), so the
-//     two wavefronts that share a SIMD run in ANTI-PHASE: every key block is four phases - GEMM 1 (MFMA), softmax
-//     (VALU), GEMM 2 (MFMA), merge (VALU) - separated by workgroup barriers, and wavefronts 4..7 run one phase behind
-//     wavefronts 0..3, so an MFMA phase of one always overlaps a VALU phase of the other on the same SIMD;
-//   * the softmax is written for instruction count: exp in the base-2 domain with every scale folded into one fma,
-//     v_max3 on the raw accumulators for the row maximum, P converted two at a time by v_cvt_pknorm_i16_f32 and packed
-//     by v_perm_b32, the int32 accumulators of both GEMMs start at the bit pattern of a float (an MFMA inline constant)
-//     so that they can be read as floats without a convert, the running O is only rescaled when a row maximum jumps by more than
-//     2^kLazyLog2, and O is normalised once, in the epilogue.
+//   * K and V tiles of 128 keys go HBM -> LDS directly (global_load_lds_dwordx4, no VGPR staging, no ds_write) into
+//     a ring of four stages, fetched three key blocks ahead, as [key][d] with the 16-byte chunk index XOR-swizzled by
+//     the row (the swizzle is applied to the global address each lane fetches), so that the 128-bit operand reads of
+//     K and the transposing reads of V (ds_read_b64_tr_b8) are bank-conflict free; Q goes once per workgroup straight
+//     into MFMA operand registers;
+//   * the kernel is bound by the instruction issue port of the SIMD (a VALU instruction holds it for 4.5 to 9 cycles,
+//     an MFMA for about 15), so the two wavefronts that share a SIMD run in ANTI-PHASE: every key block is an MFMA phase
+//     - GEMM 2 and merge of the previous block, then GEMM 1 of this one, with the merge and the row maximum issued in
+//     the shadow of the MFMAs - and a VALU phase, the softmax; workgroup barriers separate the phases, wavefronts 4..7
+//     run one phase behind wavefronts 0..3, and the wavefront in its MFMA phase runs at raised priority, so that the
+//     MFMA pipe never waits for an issue slot;
+//   * the softmax is written for instruction count and issue order: exp in the base-2 domain with every scale folded
+//     into one fma, v_max3 on the raw accumulators for the row maximum, P converted two at a time by
+//     v_cvt_pknorm_i16_f32 and packed by v_perm_b32, every exponential followed by instructions that do not need the
+//     transcendental unit, the int32 accumulators of both GEMMs started at the bit pattern of a float (an MFMA inline
+//     constant) so that they can be read as floats without a convert, the running O only rescaled when a row maximum
+//     jumps by more than 2^kLazyLog2, and O normalised once, in the epilogue.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -37,6 +40,7 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 constexpr int kBlockQ = 256;   // query rows per workgroup
 constexpr int kBlockK = 128;   // keys per softmax block (the reference's BASE_SEQ_LEN, src/fmha_i8.cu:61-95)
 constexpr int kThreads = 512;  // 8 wavefronts: 0..3 and 4..7 run the key-block phases one phase apart
+constexpr int kStages = 4;     // K/V tiles resident in LDS per kind: a tile is fetched several phases before its first use
 constexpr int kXcds = 8;
 constexpr int kMaxKeyBlocks = 512;       // seq_len <= 65536
 constexpr float kMagic = 12582912.0f;    // 1.5 * 2^23: kMagic + y holds rne(y) in its low mantissa bits (output rounding)
@@ -118,7 +122,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   constexpr int kDSteps = D / 32;                     // MFMA k-steps of GEMM 1, and 32-row output tiles of GEMM 2
   constexpr int kKeyTiles = kBlockK / 32;
 
-  __shared__ __attribute__((aligned(1024))) int8_t lds[2][2][kTileBytes];  // [buffer][K|V][tile]
+  __shared__ __attribute__((aligned(1024))) int8_t lds[kStages][2][kTileBytes];  // [stage][K|V][tile]; tile j -> stage j % kStages
   __shared__ unsigned char lds_class[kMaxKeyBlocks];  // per key block: bit0 = some key masked, bit1 = all keys masked
 
   const int tid = threadIdx.x;
@@ -180,19 +184,21 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #pragma unroll
     for (int it = 0; it < kRegionsPerWave; ++it) {
       const int region = it * kWaves + wave;
-      const unsigned dst = lds_base + (unsigned)(((kb & 1) * 2 + which) * kTileBytes + region * 1024);
+      const unsigned dst = lds_base + (unsigned)(((kb & (kStages - 1)) * 2 + which) * kTileBytes + region * 1024);
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                    :: "s"(dst), "v"(goff + region * 1024), "s"(gp) : "memory");
     }
   };
   auto issue_k = [&](int kb) { issue_tile(kg, kb, 0, ld_goff_k); };
   auto issue_v = [&](int kb) { issue_tile(vg, kb, 1, ld_goff_v); };
-  // Every wavefront issues its loads in the order K0 V0 K1 V1 K2 V2 ..., kRegionsPerWave per tile, and memory reads
-  // return in order: waiting until at most `2 tiles` of this wavefront's loads are outstanding retires everything up to
-  // and including the tile that is two tiles older than the newest one.
-  auto wait_all_but_two_tiles = [&]() {
-    if (kRegionsPerWave == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+  // Memory reads return in issue order: waiting until at most `tiles` tiles of this wavefront's loads are outstanding
+  // retires every tile older than the newest `tiles` ones.
+  auto wait_all_but = [&](int tiles) {
+    if (tiles >= 4) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(4 * kRegionsPerWave) : "memory");
+    else if (tiles == 3) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(3 * kRegionsPerWave) : "memory");
+    else if (tiles == 2) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * kRegionsPerWave) : "memory");
+    else if (tiles == 1) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kRegionsPerWave) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   };
   auto wait_all = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
   auto barrier = [&]() { asm volatile("s_barrier" ::: "memory"); };
@@ -200,7 +206,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // Loads of the prologue, all issued before any is waited for and all by inline assembly, so that every wait is an
   // explicit s_waitcnt vmcnt(n) that counts the loads still allowed in flight (memory reads return in issue order):
   //   mask bytes of the first 2048 keys (1 load) | K0 | Q (kDSteps loads) | V0
-  // (K1 and V1 follow right after the first barrier: the CU's vector memory path moves 64 bytes per cycle, and
+  // (the next tiles follow right after the first barrier: the CU's vector memory path moves 64 bytes per cycle, and
   // everything queued here delays the first GEMM.)
   const int row0 = qb * kBlockQ + wave * 32;  // first query row of this wavefront
   const bool active = row0 < S;               // seq_len is a multiple of 128, not of 256: the last workgroup may be half empty
@@ -277,31 +283,24 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   float l_blk = 0.f;    // sum of (128/32767) p over this lane's keys
 
   // Row maximum of one finished 32-key tile, folded into two independent chains (integer compare: monotone in the
-  // score, also for the biased bit patterns).
-  auto tile_max = [&](const v16i& a, int (&mx)[2], bool first) {
-    if (first) {
+  // score, also for the biased bit patterns).  Four pieces of two instructions, one behind each MFMA of the next tile.
+  auto tile_max_piece = [&](const v16i& a, int (&mx)[2], bool first, int j) {
+    if (first && j == 0) {
       mx[0] = max(max(a[0], a[1]), a[2]);
       mx[1] = max(max(a[8], a[9]), a[10]);
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        mx[0] = max(max(mx[0], a[3 + 2 * j]), a[4 + 2 * j]);
-        mx[1] = max(max(mx[1], a[11 + 2 * j]), a[12 + 2 * j]);
-      }
-      mx[0] = max(mx[0], a[7]);
-      mx[1] = max(mx[1], a[15]);
+    } else if (first) {
+      mx[0] = (j < 3) ? max(max(mx[0], a[1 + 2 * j]), a[2 + 2 * j]) : max(mx[0], a[7]);
+      mx[1] = (j < 3) ? max(max(mx[1], a[9 + 2 * j]), a[10 + 2 * j]) : max(mx[1], a[15]);
     } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        mx[0] = max(max(mx[0], a[2 * j]), a[2 * j + 1]);
-        mx[1] = max(max(mx[1], a[8 + 2 * j]), a[9 + 2 * j]);
-      }
+      mx[0] = max(max(mx[0], a[2 * j]), a[2 * j + 1]);
+      mx[1] = max(max(mx[1], a[8 + 2 * j]), a[9 + 2 * j]);
     }
   };
 
   // GEMM 1: S^T[key][query] = K . Q^T, int32 (inc/fmha_i8.cuh:120-172), one 32-key tile after the other; the row
   // maximum of tile t-1 is taken while the MFMAs of tile t run.  mx covers tiles 0 .. kKeyTiles-2 on return.
   auto phase_gemm1 = [&](int kb, v16i (&acc)[kKeyTiles], int (&mx)[2]) {
-    const int8_t* lds_k = &lds[kb & 1][0][0];
+    const int8_t* lds_k = &lds[kb & (kStages - 1)][0][0];
     const v16i zero_c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     v4i ka[2][kDSteps];  // operand reads run one key tile ahead of the MFMAs that consume them
 #pragma unroll
@@ -315,14 +314,16 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int kk = 0; kk < kDSteps; ++kk)
+      for (int kk = 0; kk < kDSteps; ++kk) {
         acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ka[t & 1][kk], qreg[kk],
                                                        kk == 0 ? (BIAS ? base_c : zero_c) : acc[t], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      if (t >= 1) {
-        tile_max(acc[t - 1], mx, t == 1);
-        asm volatile("" : "+v"(mx[0]), "+v"(mx[1]));  // keeps these few instructions here, in the shadow of the MFMAs
         __builtin_amdgcn_sched_barrier(0);
+        if (t >= 1) {
+#pragma unroll
+          for (int j = kk * 4 / kDSteps; j < (kk + 1) * 4 / kDSteps; ++j) tile_max_piece(acc[t - 1], mx, t == 1, j);
+          asm volatile("" : "+v"(mx[0]), "+v"(mx[1]));  // keeps these few instructions here, in the shadow of the MFMA
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     }
   };
@@ -332,7 +333,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     auto sf = [&](int t, int r) -> float { return BIAS ? __int_as_float(acc[t][r]) : (float)acc[t][r]; };
     l_blk = 0.f;
     if (cls == 0) {
-      tile_max(acc[kKeyTiles - 1], mx, false);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) tile_max_piece(acc[kKeyTiles - 1], mx, false, j);
       const int ti = half_max(max(mx[0], mx[1]));
       const float top = BIAS ? __int_as_float(ti) : (float)ti;
       // off = top*c2 rounded; p' = exp2(s*c2 - off) = p * 2^(resid) with one row-wide resid below 1 ulp of off, and the
@@ -427,40 +429,12 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     }
   };
 
-  // GEMM 2: O~^T[d][query] = V^T . P^T, int32 (inc/fmha_i8.cuh:255-296); accumulators start at kBaseBits
-  auto phase_gemm2 = [&](int kb, const v4i (&pk)[kKeyTiles], v16i (&oacc)[kDSteps]) {
-    const int8_t* lds_v = &lds[kb & 1][1][0];
-    typedef v2i __attribute__((address_space(3))) * lds_v2i_ptr;
-    v2i va[2][kDSteps][2];  // transposed V operands, one 32-key tile ahead of the MFMAs
-#pragma unroll
-    for (int u = 0; u < kDSteps; ++u) {
-      va[0][u][0] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u]));
-      va[0][u][1] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u] + 16 * D));
-    }
-#pragma unroll
-    for (int t = 0; t < kKeyTiles; ++t) {
-      if (t + 1 < kKeyTiles) {
-#pragma unroll
-        for (int u = 0; u < kDSteps; ++u) {
-          va[(t + 1) & 1][u][0] =
-              __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u] + 32 * (t + 1) * D));
-          va[(t + 1) & 1][u][1] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-              (lds_v2i_ptr)(lds_v + v_read_off[u] + 32 * (t + 1) * D + 16 * D));
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int u = 0; u < kDSteps; ++u) {
-        const v4i a = {va[t & 1][u][0][0], va[t & 1][u][0][1], va[t & 1][u][1][0], va[t & 1][u][1][1]};
-        oacc[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, pk[t], t == 0 ? base_c : oacc[u], 0, 0, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-
-  // online merge, normalisation deferred to the epilogue (inc/fmha_i8.cuh:298-315).  O and l are kept relative to
-  // 2^m_ref; m_ref only moves when some row's block maximum exceeds it by 2^kLazyLog2.
-  auto phase_merge = [&](const v16i (&oacc)[kDSteps]) {
+  // GEMM 2 and the online merge in one phase.  O~^T[d][query] = V^T . P^T, int32 (inc/fmha_i8.cuh:255-296), one
+  // 32-row output tile u after the other (accumulators start at kBaseBits), and tile u-1 is merged into the running O
+  // (inc/fmha_i8.cuh:298-315) four elements behind each MFMA of tile u.  Normalisation is deferred to the epilogue:
+  // O and l are kept relative to 2^m_ref, and m_ref only moves when some row's block maximum exceeds it by
+  // 2^kLazyLog2.
+  auto phase_gemm2_merge = [&](int kb, const v4i (&pk)[kKeyTiles]) {
     if (__ballot(m_blk > m_ref + kLazyLog2) != 0) {
       const float m_new = fmaxf(m_ref, m_blk);
       const float keep = __builtin_amdgcn_exp2f(m_ref - m_new);
@@ -477,88 +451,126 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     if (FASTACC) t_run += take;
     float neg_take = -take;  // P carries the sign: P = -128 p (inc/fmha_i8.cuh:298)
     asm volatile("" : "+v"(neg_take));  // a plain register operand: as a source modifier it would force the 64-bit encoding
+    auto merge_piece = [&](const v16i& oa, int u, int j) {  // four of the sixteen elements of output tile u
 #pragma unroll
-    for (int u = 0; u < kDSteps; ++u)
+      for (int r = 4 * j; r < 4 * j + 4; ++r)
+        o_f[u][r] = __builtin_fmaf(neg_take, FASTACC ? __int_as_float(oa[r]) : __int_as_float(oa[r]) - kBase, o_f[u][r]);
+    };
+
+    const int8_t* lds_v = &lds[kb & (kStages - 1)][1][0];
+    typedef v2i __attribute__((address_space(3))) * lds_v2i_ptr;
+    v2i va[2][kKeyTiles][2];  // transposed V operands of one output tile (all key tiles), one output tile ahead
+    v16i oacc[2];
+    auto read_tile = [&](int u) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        o_f[u][r] = __builtin_fmaf(neg_take, FASTACC ? __int_as_float(oacc[u][r]) : __int_as_float(oacc[u][r]) - kBase,
-                                   o_f[u][r]);
+      for (int t = 0; t < kKeyTiles; ++t) {
+        va[u & 1][t][0] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u] + 32 * t * D));
+        va[u & 1][t][1] =
+            __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u] + 32 * t * D + 16 * D));
+      }
+    };
+    read_tile(0);
+#pragma unroll
+    for (int u = 0; u < kDSteps; ++u) {
+      if (u + 1 < kDSteps) read_tile(u + 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int t = 0; t < kKeyTiles; ++t) {
+        const v4i a = {va[u & 1][t][0][0], va[u & 1][t][0][1], va[u & 1][t][1][0], va[u & 1][t][1][1]};
+        oacc[u & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, pk[t], t == 0 ? base_c : oacc[u & 1], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (u >= 1) {
+          merge_piece(oacc[(u - 1) & 1], u - 1, t);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) merge_piece(oacc[(kDSteps - 1) & 1], kDSteps - 1, j);
   };
 
   // ---- the tick schedule -------------------------------------------------------------------------------------------
-  // A tick is the interval between two workgroup barriers.  In tick T wavefronts 0..3 run phase T mod 4 of key block
-  // T div 4 (GEMM 1, softmax, GEMM 2, merge) and wavefronts 4..7 run phase (T-1) mod 4 of block (T-1) div 4.
-  // Tiles: K(j), V(j) live in buffer j mod 2.  K(j) is read in ticks 4j and 4j+1, V(j) in ticks 4j+2 and 4j+3, so
-  // K(j+2) may be fetched after barrier 4j+2 and V(j+2) after barrier 4j+4; every wavefront issues its share in the
-  // order K0 V0 K1 V1 K2 ..., K(j) must have landed before barrier 4j and V(j) before barrier 4j+2.
+  // A tick is the interval between two workgroup barriers.  Every key block i is two phases per wavefront: an MFMA
+  // phase M(i) = [GEMM 2 + merge of block i-1][GEMM 1 of block i], bound by LDS operand reads, and a VALU phase
+  // Y(i) = softmax of block i.  Wavefronts 0..3 run M(i) in tick 2i and Y(i) in tick 2i+1; wavefronts 4..7 run one tick
+  // behind, so the MFMA phase of one always overlaps the VALU phase of the other wavefront of the same SIMD.
+  // Tiles: K(j), V(j) live in stage j mod 4; K(j) is read in ticks 2j and 2j+1, V(j) in ticks 2j+2 and 2j+3, and
+  // barrier 2m publishes K(m) and V(m-1).  A wavefront is held for hundreds of cycles when it issues loads (the CU's
+  // vector memory path takes 64 bytes per cycle and all eight wavefronts queue up), so it issues at the END of its
+  // softmax phase, the one place where it would otherwise reach the barrier early: K(i+3) and V(i+2) after Y(i).  Both
+  // stages were last read in tick 2i-1.  Issue order per wavefront: K0 V0 | K1 K2 V1 | K3 V2 | K4 V3 | ...
   const int n = kb_end;
   auto cls_of = [&](int kb) { return __builtin_amdgcn_readfirstlane((int)lds_class[kb]); };
-  auto wait_tile = [&](bool newer_in_flight) { if (newer_in_flight) wait_all_but_two_tiles(); else wait_all(); };
+  auto works = [&](int kb) { return active && !(cls_of(kb) & 2); };  // nothing in a fully masked block is attended to
+  auto issue_first = [&]() {          // after barrier 0
+    if (n > 1) issue_k(1);
+    if (n > 2) issue_k(2);
+    if (n > 1) issue_v(1);
+  };
+  auto issue_after_softmax = [&](int i) {
+    if (i + 3 < n) issue_k(i + 3);
+    if (i + 2 < n) issue_v(i + 2);
+  };
+  // Before barrier 2m every wavefront waits for its share of K(m) and V(m-1).  Tiles issued later may stay in flight:
+  // K(m+1), V(m) (after Y(m-2)) and, for the wavefronts that have already finished Y(m-1), K(m+2), V(m+1).
+  auto wait_tiles_for = [&](int m, bool after_next_softmax) {
+    int newer = (m + 1 < n ? 1 : 0) + (m < n ? 1 : 0);
+    if (after_next_softmax) newer += (m + 2 < n ? 1 : 0) + (m + 1 < n ? 1 : 0);
+    wait_all_but(newer);
+  };
+  v16i acc[kKeyTiles];  // S^T of the block whose softmax comes next (GEMM 1 -> softmax, across a barrier)
+  int mx[2];
+  // Where GEMM 1 is skipped the old scores are dead; saying so (an empty definition) keeps 64 registers from being
+  // carried through the following MFMA phase.
+  auto forget_scores = [&]() {
+#pragma unroll
+    for (int t = 0; t < kKeyTiles; ++t) asm volatile("" : "=v"(acc[t]));
+    asm volatile("" : "=v"(mx[0]), "=v"(mx[1]));
+  };
+  // The wavefront in its MFMA phase gets the issue slots it asks for: an MFMA, an operand read or a merge instruction
+  // that waits behind the other wavefront's softmax stream leaves the MFMA pipe idle, the reverse costs nothing.
+  auto raise_priority = [&]() { asm volatile("s_setprio 3" ::: "memory"); };
+  auto drop_priority = [&]() { asm volatile("s_setprio 0" ::: "memory"); };
+  barrier();                                   // barrier 0 (K(0) landed: prologue)
   if (wave < 4) {
-    for (int i = 0; i < n; ++i) {
-      const int cls = cls_of(i);
-      const bool work = active && !(cls & 2);  // nothing in a fully masked block is attended to
-      if (i > 0) wait_tile(i + 1 < n);         // K(i) landed (V(i), K(i+1) may still be in flight); K(0): prologue
-      barrier();                               // barrier 4i
-      if (i + 1 < n) {
-        if (i == 0) issue_k(1);
-        issue_v(i + 1);
-      }
-      if (work) {
-        v16i acc[kKeyTiles];
-        v4i pk[kKeyTiles];
-        v16i oacc[kDSteps];
-        int mx[2];
-        phase_gemm1(i, acc, mx);
-        barrier();                             // barrier 4i+1
-        phase_softmax(i, cls, acc, pk, mx);
-        wait_tile(i + 1 < n);                  // V(i) landed
-        barrier();                             // barrier 4i+2
-        if (i + 2 < n) issue_k(i + 2);
-        phase_gemm2(i, pk, oacc);
-        barrier();                             // barrier 4i+3
-        phase_merge(oacc);
-      } else {
-        barrier();
-        wait_tile(i + 1 < n);
-        barrier();
-        if (i + 2 < n) issue_k(i + 2);
-        barrier();
-      }
-    }
-    barrier();                                 // barrier 4n: wavefronts 4..7 run their last merge
-  } else {
-    barrier();                                 // barrier 0 (K(0) landed: prologue)
-    if (n > 1) { issue_k(1); issue_v(1); }
+    if (n > 0 && works(0)) phase_gemm1(0, acc, mx);
+    else forget_scores();
+    issue_first();
     for (int i = 0; i < n; ++i) {
       const int cls = cls_of(i);
       const bool work = active && !(cls & 2);
-      barrier();                               // barrier 4i+1
-      if (work) {
-        v16i acc[kKeyTiles];
-        v4i pk[kKeyTiles];
-        v16i oacc[kDSteps];
-        int mx[2];
-        phase_gemm1(i, acc, mx);
-        wait_tile(i + 1 < n);                  // V(i) landed
-        barrier();                             // barrier 4i+2
-        if (i + 2 < n) issue_k(i + 2);
-        phase_softmax(i, cls, acc, pk, mx);
-        barrier();                             // barrier 4i+3
-        phase_gemm2(i, pk, oacc);
-        wait_tile(i + 2 < n);                  // K(i+1) landed
-        barrier();                             // barrier 4(i+1)
-        if (i + 2 < n) issue_v(i + 2);
-        phase_merge(oacc);
-      } else {
-        wait_tile(i + 1 < n);
-        barrier();
-        if (i + 2 < n) issue_k(i + 2);
-        barrier();
-        wait_tile(i + 2 < n);
-        barrier();
-        if (i + 2 < n) issue_v(i + 2);
-      }
+      v4i pk[kKeyTiles];
+      barrier();                               // barrier 2i+1
+      if (work) phase_softmax(i, cls, acc, pk, mx);
+      issue_after_softmax(i);
+      wait_tiles_for(i + 1, true);
+      barrier();                               // barrier 2i+2
+      raise_priority();
+      if (work) phase_gemm2_merge(i, pk);
+      if (i + 1 < n && works(i + 1)) phase_gemm1(i + 1, acc, mx);
+      else forget_scores();
+      drop_priority();
+    }
+    barrier();                                 // barrier 2n+1: wavefronts 4..7 run their last MFMA phase after it
+  } else {
+    issue_first();
+    barrier();                                 // barrier 1
+    if (n > 0 && works(0)) phase_gemm1(0, acc, mx);
+    else forget_scores();
+    for (int i = 0; i < n; ++i) {
+      const int cls = cls_of(i);
+      const bool work = active && !(cls & 2);
+      v4i pk[kKeyTiles];
+      wait_tiles_for(i + 1, false);
+      barrier();                               // barrier 2i+2
+      if (work) phase_softmax(i, cls, acc, pk, mx);
+      issue_after_softmax(i);
+      barrier();                               // barrier 2i+3
+      raise_priority();
+      if (work) phase_gemm2_merge(i, pk);
+      if (i + 1 < n && works(i + 1)) phase_gemm1(i + 1, acc, mx);
+      else forget_scores();
+      drop_priority();
     }
   }
   wait_all();  // nothing may still be writing LDS when the wavefront ends (only possible when every key is masked)
