@@ -15,12 +15,14 @@
  *   asynchrony     one kernel is enqueued on `stream`; the call returns immediately and never synchronises.
  *   threading      no mutable global state: callable concurrently from any host thread.
  *
- * Supported shapes: head_dim in {64, 128}; seq_len a positive multiple of 128, at most 65536; batch_num, head_num >= 1.
- * (The reference's ladder, src/fmha_i8.cu:39-154, covers head_dim in {64,128} and eleven fixed seq_len values;
- * every one of its 128-multiples is covered here, and so is any other multiple of 128.)
+ * Supported shapes: head_dim in {64, 128}; seq_len a positive multiple of 64, at most 65536; batch_num, head_num >= 1.
+ * (The reference's ladder, src/fmha_i8.cu:39-154, covers head_dim in {64,128} and eleven fixed seq_len values: 64, 128,
+ * 192, 256, 320, 384, 448, 512, 1024, 2048, 4096.  All of them are covered here, and so is every other multiple of 64.
+ * As in the reference, the softmax works on blocks of 128 keys when seq_len is a multiple of 128 and on blocks of 64 keys
+ * otherwise - the block size is part of the numerics, because P is quantised against the BLOCK-LOCAL row maximum.)
  *
  * Numerics follow the reference kernel (inc/fmha_i8.cuh:71-72,181-253,298-332): int32 Q.K^T, 1/sqrt(d) and
- * q_amax*k_amax/127^2 dequantisation, softmax over blocks of 128 keys with the BLOCK-LOCAL row maximum,
+ * q_amax*k_amax/127^2 dequantisation, softmax over blocks of 128 (or 64) keys with the BLOCK-LOCAL row maximum,
  * P requantised to int8 in [-128, 0] with scale -128, int32 P.V, online (m, l, O) merge, O requantised with
  * v_amax/(128*o_amax), round-half-even, clamp to [-127, 127].  Rows whose keys are all masked produce 0.
  */
@@ -38,7 +40,7 @@ extern "C" {
 #define FMHA_I8_OK 0
 #define FMHA_I8_ERR_NULL_POINTER 1   /* q, k, v, padding_mask or o is NULL */
 #define FMHA_I8_ERR_HEAD_DIM 2       /* head_dim not in {64, 128} */
-#define FMHA_I8_ERR_SEQ_LEN 3        /* seq_len <= 0, not a multiple of 128, or > 65536 */
+#define FMHA_I8_ERR_SEQ_LEN 3        /* seq_len <= 0, not a multiple of 64, or > 65536 */
 #define FMHA_I8_ERR_BATCH_HEAD 4     /* batch_num or head_num <= 0, or the grid would exceed HIP limits */
 #define FMHA_I8_ERR_ALIGNMENT 5      /* q, k, v or o not 16-byte aligned */
 #define FMHA_I8_ERR_SCALE 6          /* an amax is not finite, or o_amax <= 0 */

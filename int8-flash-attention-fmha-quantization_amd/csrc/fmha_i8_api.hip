@@ -17,8 +17,7 @@ int check_args(const FMHAParamI8& p, const AttnDataDescriptor& a, const void* q,
                const void* mask, const void* o) {
   if (!q || !k || !v || !mask || !o) return FMHA_I8_ERR_NULL_POINTER;
   if (a.head_dim != 64 && a.head_dim != 128) return FMHA_I8_ERR_HEAD_DIM;
-  if (a.seq_len <= 0 || a.seq_len % fmha_i8_gfx950::kBlockK != 0 ||
-      a.seq_len > fmha_i8_gfx950::kBlockK * fmha_i8_gfx950::kMaxKeyBlocks)
+  if (a.seq_len <= 0 || a.seq_len % fmha_i8_gfx950::kBlockKSmall != 0 || a.seq_len > 65536)
     return FMHA_I8_ERR_SEQ_LEN;
   if (a.batch_num <= 0 || a.head_num <= 0) return FMHA_I8_ERR_BATCH_HEAD;
   const long long wgs = (long long)a.batch_num * a.head_num * ((a.seq_len + fmha_i8_gfx950::kBlockQ - 1) / fmha_i8_gfx950::kBlockQ);
@@ -28,6 +27,15 @@ int check_args(const FMHAParamI8& p, const AttnDataDescriptor& a, const void* q,
   if (!isfinite(p.q_amax) || !isfinite(p.k_amax) || !isfinite(p.v_amax) || !isfinite(p.o_amax) || !(p.o_amax > 0.f))
     return FMHA_I8_ERR_SCALE;
   return FMHA_I8_OK;
+}
+
+template <int D, int BK>
+void launch_variant(bool bias, bool fast, dim3 grid, dim3 block, hipStream_t stream, const fmha_i8_gfx950::KernelArgs& args) {
+  using namespace fmha_i8_gfx950;
+#define FMHA_LAUNCH(BB, FF) hipLaunchKernelGGL((fmha_i8_fwd_kernel<D, BK, BB, FF>), grid, block, 0, stream, args)
+  if (bias) { if (fast) FMHA_LAUNCH(true, true); else FMHA_LAUNCH(true, false); }
+  else { if (fast) FMHA_LAUNCH(false, true); else FMHA_LAUNCH(false, false); }
+#undef FMHA_LAUNCH
 }
 
 int launch(hipStream_t stream, const FMHAParamI8& p, const AttnDataDescriptor& a, const void* q, const void* k,
@@ -61,18 +69,18 @@ int launch(hipStream_t stream, const FMHAParamI8& p, const AttnDataDescriptor& a
   // Folding the accumulator offset into the running O (see FASTACC in the kernel) costs a rounding of relative size
   // 2^-24 at magnitude kBase * sum(take) per key block; normalised by the row sum (>= sum(take)) and scaled to output
   // LSBs that is at most about 0.0034 * (v_amax/o_amax) * sqrt(key blocks).  Take it while that stays below 0.1 LSB.
-  const float lsb_bound = 0.0034f * fabsf(p.v_amax / p.o_amax) * sqrtf((float)(a.seq_len / fmha_i8_gfx950::kBlockK));
+  // Blocks of 128 keys, as the reference uses for its multiples of 128; its other lengths (64, 192, 320, 448:
+  // src/fmha_i8.cu:41-60) run in blocks of 64 keys, and so does every other odd multiple of 64 here.
+  const int block_keys = a.seq_len % fmha_i8_gfx950::kBlockK == 0 ? fmha_i8_gfx950::kBlockK : fmha_i8_gfx950::kBlockKSmall;
+  const float lsb_bound = 0.0034f * fabsf(p.v_amax / p.o_amax) * sqrtf((float)(a.seq_len / block_keys));
   const bool fast = lsb_bound < 0.1f;
-  using namespace fmha_i8_gfx950;
-#define FMHA_LAUNCH(DD, BB, FF) hipLaunchKernelGGL((fmha_i8_fwd_kernel<DD, BB, FF>), grid, block, 0, stream, args)
   if (a.head_dim == 128) {
-    if (bias) { if (fast) FMHA_LAUNCH(128, true, true); else FMHA_LAUNCH(128, true, false); }
-    else { if (fast) FMHA_LAUNCH(128, false, true); else FMHA_LAUNCH(128, false, false); }
+    if (block_keys == fmha_i8_gfx950::kBlockK) launch_variant<128, fmha_i8_gfx950::kBlockK>(bias, fast, grid, block, stream, args);
+    else launch_variant<128, fmha_i8_gfx950::kBlockKSmall>(bias, fast, grid, block, stream, args);
   } else {
-    if (bias) { if (fast) FMHA_LAUNCH(64, true, true); else FMHA_LAUNCH(64, true, false); }
-    else { if (fast) FMHA_LAUNCH(64, false, true); else FMHA_LAUNCH(64, false, false); }
+    if (block_keys == fmha_i8_gfx950::kBlockK) launch_variant<64, fmha_i8_gfx950::kBlockK>(bias, fast, grid, block, stream, args);
+    else launch_variant<64, fmha_i8_gfx950::kBlockKSmall>(bias, fast, grid, block, stream, args);
   }
-#undef FMHA_LAUNCH
   const hipError_t err = hipGetLastError();
   return err == hipSuccess ? FMHA_I8_OK : FMHA_I8_ERR_HIP_BASE + (int)err;
 }
@@ -105,7 +113,7 @@ const char* FMHAInferI8StatusString(int status) {
     case FMHA_I8_OK: return "ok";
     case FMHA_I8_ERR_NULL_POINTER: return "null pointer argument";
     case FMHA_I8_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
-    case FMHA_I8_ERR_SEQ_LEN: return "seq_len must be a positive multiple of 128, at most 65536";
+    case FMHA_I8_ERR_SEQ_LEN: return "seq_len must be a positive multiple of 64, at most 65536";
     case FMHA_I8_ERR_BATCH_HEAD: return "batch_num and head_num must be positive (and the grid must fit)";
     case FMHA_I8_ERR_ALIGNMENT: return "q, k, v and o must be 16-byte aligned";
     case FMHA_I8_ERR_SCALE: return "amax values must be finite and o_amax > 0";

@@ -38,11 +38,12 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kBlockQ = 256;   // query rows per workgroup
-constexpr int kBlockK = 128;   // keys per softmax block (the reference's BASE_SEQ_LEN, src/fmha_i8.cu:61-95)
+constexpr int kBlockK = 128;   // keys per softmax block (the reference's BASE_SEQ_LEN, src/fmha_i8.cu:61-95) ...
+constexpr int kBlockKSmall = 64;  // ... and for its sequence lengths that are odd multiples of 64 (src/fmha_i8.cu:41-60)
 constexpr int kThreads = 512;  // 8 wavefronts: 0..3 and 4..7 run the key-block phases one phase apart
 constexpr int kStages = 4;     // K/V tiles resident in LDS per kind: a tile is fetched several phases before its first use
 constexpr int kXcds = 8;
-constexpr int kMaxKeyBlocks = 512;       // seq_len <= 65536
+constexpr int kMaxKeyBlocks = 1024;      // seq_len <= 65536, also in blocks of 64 keys
 constexpr float kMagic = 12582912.0f;    // 1.5 * 2^23: kMagic + y holds rne(y) in its low mantissa bits (output rounding)
 // Both GEMMs start their int32 accumulators at the bit pattern of the float 1/(2 pi), which the MFMA takes as an INLINE
 // CONSTANT C operand (no registers, no moves).  That float sits 2292099 ulps above 2^-3 and 6096509 below 2^-2, more than
@@ -112,15 +113,17 @@ __device__ __forceinline__ float half_sum(float x) {
 // FASTACC: the running O absorbs the kBase offset of the GEMM 2 accumulators (one fma per element and key block
 // instead of subtract + fma) and the offset is taken out once, in the epilogue.  O then lives near kBase * sum(take)
 // and each merge rounds at that magnitude; the host enables it only where that rounding is far below one output LSB.
-template <int D, bool BIAS, bool FASTACC>
+template <int D, int BK, bool BIAS, bool FASTACC>
 __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelArgs args) {
   constexpr int kChunks = D / 16;                     // 16-byte chunks per row
-  constexpr int kTileBytes = kBlockK * D;             // one K or V tile
+  constexpr int kTileBytes = BK * D;                  // one K or V tile
   constexpr int kWaves = kThreads / 64;
-  constexpr int kRegionsPerWave = kTileBytes / 1024 / kWaves;  // 1 KiB (64 lanes x 16 B) direct-to-LDS loads per wave
+  constexpr int kRegions = kTileBytes / 1024;         // 1 KiB (64 lanes x 16 B) direct-to-LDS loads per tile
+  constexpr int kRegionsPerWave = (kRegions + kWaves - 1) / kWaves;  // ... and per wavefront (a tile of fewer regions
+                                                      // than wavefronts is loaded twice: all wavefronts count alike)
   constexpr int kRowsPerRegion = 1024 / D;
   constexpr int kDSteps = D / 32;                     // MFMA k-steps of GEMM 1, and 32-row output tiles of GEMM 2
-  constexpr int kKeyTiles = kBlockK / 32;
+  constexpr int kKeyTiles = BK / 32;
 
   __shared__ __attribute__((aligned(1024))) int8_t lds[kStages][2][kTileBytes];  // [stage][K|V][tile]; tile j -> stage j % kStages
   __shared__ unsigned char lds_class[kMaxKeyBlocks];  // per key block: bit0 = some key masked, bit1 = all keys masked
@@ -146,7 +149,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   const int8_t* __restrict__ kg = args.k + head_off;
   const int8_t* __restrict__ vg = args.v + head_off;
   const int8_t* __restrict__ mg = args.mask + (long)b * S;
-  const int n_blocks = S / kBlockK;
+  const int n_blocks = S / BK;
 
   // The prologue puts every cold miss in flight before it waits for any of them: the mask bytes, the first two K/V
   // tiles (tile 1 on speculation: it exists whenever seq_len >= 256, whether or not its keys are masked) and the Q rows.
@@ -183,7 +186,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     const int8_t* gp = gbase + (long)kb * kTileBytes;  // wave-uniform base (SGPR pair)
 #pragma unroll
     for (int it = 0; it < kRegionsPerWave; ++it) {
-      const int region = it * kWaves + wave;
+      const int region = (it * kWaves + wave) % kRegions;
       const unsigned dst = lds_base + (unsigned)(((kb & (kStages - 1)) * 2 + which) * kTileBytes + region * 1024);
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                    :: "s"(dst), "v"(goff + region * 1024), "s"(gp) : "memory");
@@ -227,7 +230,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   }
   issue_v(0);
 
-  // ---- classify the key blocks of this batch entry: 4 mask bytes per lane, two blocks per wavefront ballot ---------
+  // ---- classify the key blocks of this batch entry: 4 mask bytes per lane, BK/4 lanes per block ---------------------
   asm volatile("s_waitcnt vmcnt(%1)" : "+v"(mask_word) : "n"(2 * kRegionsPerWave + kDSteps) : "memory");
   for (int base = 0; base < S; base += 4 * kThreads) {
     const int j = base + 4 * tid;
@@ -239,9 +242,11 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       nib = (mg[j] != 0 ? 1 : 0) | (mg[j + 1] != 0 ? 2 : 0) | (mg[j + 2] != 0 ? 4 : 0) | (mg[j + 3] != 0 ? 8 : 0);
     }
     const unsigned long long some = __ballot(nib != 0), all = __ballot(nib == 15);
-    if ((lane & 31) == 0 && j < S) {
-      const unsigned half_some = (unsigned)(some >> (lane & 32)), half_all = (unsigned)(all >> (lane & 32));
-      lds_class[j / kBlockK] = (unsigned char)((half_some != 0 ? 1 : 0) | (half_all == 0xffffffffu ? 2 : 0));
+    constexpr int kLanesPerBlock = BK / 4;
+    constexpr unsigned long long kBlockBits = (1ull << kLanesPerBlock) - 1;
+    if (lane % kLanesPerBlock == 0 && j < S) {
+      const unsigned long long blk_some = (some >> lane) & kBlockBits, blk_all = (all >> lane) & kBlockBits;
+      lds_class[j / BK] = (unsigned char)((blk_some != 0 ? 1 : 0) | (blk_all == kBlockBits ? 2 : 0));
     }
   }
   __syncthreads();
@@ -392,7 +397,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       l_blk = half_sum(l_blk);
     } else {
       // some keys of this block are masked out (nonzero mask byte, inc/fmha_i8.cuh:189-192,216-221)
-      const int8_t* mp = mg + kb * kBlockK + 4 * i32;
+      const int8_t* mp = mg + kb * BK + 4 * (i32 % (BK / 4));  // lanes past the block re-read it; their bits are not used
       const int nib = (mp[0] != 0 ? 1 : 0) | (mp[1] != 0 ? 2 : 0) | (mp[2] != 0 ? 4 : 0) | (mp[3] != 0 ? 8 : 0);
       unsigned mbits[kKeyTiles];  // bit 4a+bb of mbits[t] <-> key 32t + 8a + 4g + bb
 #pragma unroll
@@ -480,7 +485,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         oacc[u & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, pk[t], t == 0 ? base_c : oacc[u & 1], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         if (u >= 1) {
-          merge_piece(oacc[(u - 1) & 1], u - 1, t);
+#pragma unroll
+          for (int j = t * 4 / kKeyTiles; j < (t + 1) * 4 / kKeyTiles; ++j) merge_piece(oacc[(u - 1) & 1], u - 1, j);
           __builtin_amdgcn_sched_barrier(0);
         }
       }

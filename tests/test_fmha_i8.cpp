@@ -5,7 +5,7 @@
 // as the reference's driver calls gpuImpl::FMHAInferI8 (test_fmha_i8.cpp:204-222).
 //
 //   test_fmha_i8 --config 3                 one of the five benchmark configurations
-//   test_fmha_i8 --sweep                    the reference's own sweep: B=H=1, S in {128..4096 step per its list}, d in {64,128},
+//   test_fmha_i8 --sweep                    the reference's own sweep: B=H=1, S in {64,128,...,512,1024,2048,4096}, d in {64,128},
 //                                           uniform(+-0.5) Q/K, |uniform| V, scattered 20 % mask, o_amax measured
 //   test_fmha_i8 --B 2 --H 4 --S 512 --d 64 [--valid L] [--dist normal|student_t|reference]
 //   common: --seed N --iters N --warmup N --cpu-heads N (0 = all) --cpu-threads N --json FILE --no-check
@@ -226,7 +226,7 @@ bool run_case(const Case& c, const Options& opt, FILE* json) {
     std::vector<int8_t> want(n, 0);
     auto t0 = std::chrono::steady_clock::now();
     fmha_oracle::fmha_i8_cpu_blockwise(t.q.data(), t.k.data(), t.v.data(), t.mask.data(), want.data(), c.B, c.H, c.S,
-                                       c.d, t.q_amax, t.k_amax, t.v_amax, o_amax, 128, threads, 0, cpu_heads);
+                                       c.d, t.q_amax, t.k_amax, t.v_amax, o_amax, c.S % 128 == 0 ? 128 : 64, threads, 0, cpu_heads);
     cpu_i8_s = seconds_since(t0);
     const long m = cpu_heads * c.S * c.d;
     int worst = 0;
@@ -280,8 +280,8 @@ int main(int argc, char** argv) {
     };
     if (a == "--config") cases.push_back(config_case(atoi(val())));
     else if (a == "--sweep") {
-      // test_fmha_i8.cpp:295-309, restricted to the multiples of 128 this library offers
-      for (int S : {128, 256, 384, 512, 1024, 2048, 4096})
+      // test_fmha_i8.cpp:295-309: every length of the launch ladder (src/fmha_i8.cu:39-154)
+      for (int S : {64, 128, 192, 256, 320, 384, 448, 512, 1024, 2048, 4096})
         for (int d : {64, 128}) {
           Case c;
           c.name = "sweep", c.B = 1, c.H = 1, c.S = S, c.d = d, c.dist = "reference", c.pad = "scatter";

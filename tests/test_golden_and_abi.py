@@ -61,9 +61,11 @@ def test_argument_checks_need_no_gpu(pkg):
     for d in (0, 32, 96, 256):
         assert pkg.FMHAInferI8CheckArgs(P, pkg.AttnDataDescriptor(1, 128, 1, d), a16, a16, a16, a16, a16) == \
             pkg.FMHA_I8_ERR_HEAD_DIM
-    for s in (0, -128, 64, 192, 1000):  # the reference's 64-multiples (src/fmha_i8.cu:41-60) are not offered
+    for s in (0, -128, 32, 100, 1000, 65600):
         assert pkg.FMHAInferI8CheckArgs(P, pkg.AttnDataDescriptor(1, s, 1, 64), a16, a16, a16, a16, a16) == \
             pkg.FMHA_I8_ERR_SEQ_LEN
+    for s in (64, 128, 192, 320, 448, 512, 4096, 65536):  # every length of the reference's ladder (src/fmha_i8.cu:39-154)
+        assert pkg.FMHAInferI8CheckArgs(P, pkg.AttnDataDescriptor(1, s, 1, 64), a16, a16, a16, a16, a16) == pkg.FMHA_I8_OK
     assert pkg.FMHAInferI8CheckArgs(P, pkg.AttnDataDescriptor(0, 128, 1, 64), a16, a16, a16, a16, a16) == \
         pkg.FMHA_I8_ERR_BATCH_HEAD
     assert pkg.FMHAInferI8CheckArgs(pkg.FMHAParamI8(1, 1, 1, 0.0), ok, a16, a16, a16, a16, a16) == pkg.FMHA_I8_ERR_SCALE

@@ -33,8 +33,10 @@ def gpu_run(pkg, dev, c, **scales):
 def cpu_run(orc, c, heads=None, **scales):
     s = dict(q_amax=c["q_amax"], k_amax=c["k_amax"], v_amax=c["v_amax"], o_amax=c["o_amax"])
     s.update(scales)
+    # softmax blocks of 128 keys, or of 64 for the lengths that are not multiples of 128 (src/fmha_i8.cu:41-60)
+    block = 128 if c["q"].shape[2] % 128 == 0 else 64
     return orc.fmha_i8_blockwise(c["q"], c["k"], c["v"], c["mask"], s["q_amax"], s["k_amax"], s["v_amax"], s["o_amax"],
-                                 heads=heads)
+                                 block=block, heads=heads)
 
 
 def check(got, want, what):
@@ -68,6 +70,32 @@ def test_reference_sweep(pkg, orc, dev, S, d):
     check(got, cpu_run(orc, c), "sweep S=%d d=%d" % (S, d))
     dev_pct = orc.mean_rel_deviation_pct(got, o_ref, c["o_amax"])
     assert dev_pct < 20.0, dev_pct  # inc/utils.hpp:88
+
+
+# ---- the reference's other lengths (src/fmha_i8.cu:41-60: 64, 192, 320, 448 run with 64-key softmax blocks), plus a
+# longer odd multiple of 64; unmasked, scattered mask and a padded tail that leaves whole blocks masked -------------------
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("S", [64, 192, 320, 448, 1088])
+@pytest.mark.parametrize("pad", ["none", "scatter", "tail"])
+def test_sixty_four_key_blocks(pkg, orc, dev, S, d, pad):
+    B, H = 2, 3
+    if pad == "tail":
+        c = fc.make_inputs(B, H, S, d, dist="normal", seed=77, valid_lengths=[S - 32, max(S - 160, 16)])
+    else:
+        c = fc.make_inputs(B, H, S, d, dist="normal", pad=pad, seed=77)
+    check(gpu_run(pkg, dev, c), cpu_run(orc, c), "S=%d d=%d %s" % (S, d, pad))
+
+
+def test_sixty_four_key_blocks_reference_sweep(pkg, orc, dev):
+    # the reference driver's own sweep over its 64-multiples (test_fmha_i8.cpp:295-309), reference-style data
+    for d in (64, 128):
+        for S in (64, 192, 320, 448):
+            c = fc.make_inputs(1, 1, S, d, dist="reference", pad="scatter", seed=31)
+            o_ref = orc.fmha_fp32(c["qf"], c["kf"], c["vf"], c["mask"])
+            c["o_amax"] = orc.abs_max(o_ref)
+            got = gpu_run(pkg, dev, c)
+            check(got, cpu_run(orc, c), "sweep64 S=%d d=%d" % (S, d))
+            assert orc.mean_rel_deviation_pct(got, o_ref, c["o_amax"]) < 20.0
 
 
 # ---- the five benchmark configurations -----------------------------------------------------------------------------
@@ -233,11 +261,11 @@ def test_void_entry_point_streams_and_use_tcu_flag(pkg, orc, dev):
 
 def test_unsupported_shapes_leave_output_untouched(pkg, dev):
     import torch
-    q = torch.zeros(1, 1, 192, 64, dtype=torch.int8, device=dev)
-    m = torch.zeros(1, 192, dtype=torch.int8, device=dev)
+    q = torch.zeros(1, 1, 160, 64, dtype=torch.int8, device=dev)
+    m = torch.zeros(1, 160, dtype=torch.int8, device=dev)
     o = torch.full_like(q, 55)
     P = pkg.FMHAParamI8(1, 1, 1, 1)
-    assert pkg.FMHAInferI8Status(None, P, pkg.AttnDataDescriptor(1, 192, 1, 64), q, q, q, m, o) == \
+    assert pkg.FMHAInferI8Status(None, P, pkg.AttnDataDescriptor(1, 160, 1, 64), q, q, q, m, o) == \
         pkg.FMHA_I8_ERR_SEQ_LEN
     pkg.FMHAInferI8(None, P, pkg.AttnDataDescriptor(1, 128, 1, 96), q, q, q, m, o, True)  # prints, launches nothing
     torch.cuda.synchronize()
