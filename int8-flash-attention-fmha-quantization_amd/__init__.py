@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libfmha_i8.so")
 
 EXPORTED_SYMBOLS = ("FMHAInferI8", "FMHAInferI8Status", "FMHAInferI8CheckArgs", "FMHAInferI8StatusString",
-                    "FMHAInferI8Version")
+                    "FMHAInferI8Version", "FMHAAbsMaxF32", "FMHAQuantizeI8", "FMHADequantizeI8")
 
 FMHA_I8_OK = 0
 FMHA_I8_ERR_NULL_POINTER = 1
@@ -83,6 +83,13 @@ def load_library(path=None):
     L.FMHAInferI8StatusString.restype = C.c_char_p
     L.FMHAInferI8Version.argtypes = []
     L.FMHAInferI8Version.restype = C.c_char_p
+    # include/fmha_quant.h
+    L.FMHAAbsMaxF32.argtypes = [ptr, ptr, C.c_longlong, ptr]
+    L.FMHAAbsMaxF32.restype = C.c_int
+    L.FMHAQuantizeI8.argtypes = [ptr, ptr, C.c_longlong, C.c_float, ptr, ptr]
+    L.FMHAQuantizeI8.restype = C.c_int
+    L.FMHADequantizeI8.argtypes = [ptr, ptr, C.c_longlong, C.c_float, ptr]
+    L.FMHADequantizeI8.restype = C.c_int
     if path is None:
         _lib = L
     return L
@@ -127,6 +134,55 @@ def status_string(status):
 
 def version():
     return load_library().FMHAInferI8Version().decode()
+
+
+def _check(status):
+    if status != FMHA_I8_OK:
+        raise FMHAError(status, status_string(status) if status < 1000 else "HIP error %d" % (status - 1000))
+
+
+def FMHAAbsMaxF32(stream, x, n, amax_out):
+    """abs_max (inc/utils.hpp:31-39) on the GPU: *amax_out = max |x[i]|, device pointers, status code."""
+    return int(load_library().FMHAAbsMaxF32(_stream(stream), _ptr(x), int(n), _ptr(amax_out)))
+
+
+def FMHAQuantizeI8(stream, x, n, amax_host, amax_dev, out):
+    """float_quant2_int8 (inc/utils.hpp:23-29) over n floats on the GPU; amax from device memory when amax_dev is given."""
+    return int(load_library().FMHAQuantizeI8(_stream(stream), _ptr(x), int(n), float(amax_host), _ptr(amax_dev), _ptr(out)))
+
+
+def FMHADequantizeI8(stream, x, n, amax, out):
+    """(float)x / 127 * amax (inc/utils.hpp:53) over n int8 values on the GPU."""
+    return int(load_library().FMHADequantizeI8(_stream(stream), _ptr(x), int(n), float(amax), _ptr(out)))
+
+
+def quantize_tensor(x, amax=None, stream=None):
+    """Convenience for a contiguous fp32 torch tensor on the GPU: returns (int8 tensor, amax as a 1-element device
+    tensor).  With amax=None the maximum is measured on the GPU and never visits the host."""
+    import torch
+    if not (x.is_cuda and x.dtype == torch.float32 and x.is_contiguous()):
+        raise ValueError("x must be a contiguous float32 tensor on the GPU")
+    st = stream if stream is not None else torch.cuda.current_stream(x.device)
+    out = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    if amax is None:
+        a = torch.empty(1, dtype=torch.float32, device=x.device)
+        _check(FMHAAbsMaxF32(st, x, x.numel(), a))
+        _check(FMHAQuantizeI8(st, x, x.numel(), 0.0, a, out))
+    else:
+        a = torch.full((1,), float(amax), dtype=torch.float32, device=x.device)
+        _check(FMHAQuantizeI8(st, x, x.numel(), float(amax), None, out))
+    return out, a
+
+
+def dequantize_tensor(x, amax, stream=None):
+    """int8 torch tensor on the GPU -> float32, (float)x / 127 * amax."""
+    import torch
+    if not (x.is_cuda and x.dtype == torch.int8 and x.is_contiguous()):
+        raise ValueError("x must be a contiguous int8 tensor on the GPU")
+    st = stream if stream is not None else torch.cuda.current_stream(x.device)
+    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    _check(FMHADequantizeI8(st, x, x.numel(), float(amax), out))
+    return out
 
 
 def fmha_infer_i8(q, k, v, padding_mask, q_amax, k_amax, v_amax, o_amax=1.0, out=None, stream=None):

@@ -6,9 +6,10 @@ import subprocess
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 LIB_PATH = os.path.join(HERE, "libfmha_i8.so")
-SOURCES = [os.path.join(HERE, "csrc", "fmha_i8_api.hip")]
+SOURCES = [os.path.join(HERE, "csrc", "fmha_i8_api.hip"), os.path.join(HERE, "csrc", "fmha_quant.hip")]
 DEPENDS = SOURCES + [os.path.join(HERE, "csrc", "fmha_i8_kernel.hip"),
-                     os.path.join(ROOT, "include", "fmha_i8.h"), os.path.join(ROOT, "include", "fmha_param_i8.h")]
+                     os.path.join(ROOT, "include", "fmha_i8.h"), os.path.join(ROOT, "include", "fmha_param_i8.h"),
+                     os.path.join(ROOT, "include", "fmha_quant.h")]
 # Packed-FP32 instruction selection is switched off for all device code (a flag for hipcc's device pass; the host pass
 # prints a harmless "not a recognized feature" note).
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

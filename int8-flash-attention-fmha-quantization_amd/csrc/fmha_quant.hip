@@ -1,0 +1,187 @@
+// Quantisation front end / back end of the INT8 attention path for gfx950: abs-max, fp32 -> int8, int8 -> fp32.
+// The reference does these on the host, one element at a time (inc/utils.hpp:23-39,53); here they are streaming
+// kernels whose only cost is HBM traffic: 128-bit loads, one wavefront instruction covers 1 KiB of contiguous input,
+// a few thousand wavefronts in flight, no LDS except for the block reduction of the maximum.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/fmha_quant.h"
+
+// Every float operation below must round exactly where the reference's host code rounds: no fused multiply-add.
+#pragma clang fp contract(off)
+
+namespace fmha_i8_gfx950 {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int kQuantThreads = 256;
+constexpr int kQuantUnroll = 4;          // 16-byte units per thread and loop trip: 64 B per lane in flight per trip
+constexpr int kQuantMaxBlocks = 256 * 2; // two workgroups of 4 wavefronts per CU: measured best from 32 MiB to 1 GiB (more
+                                         // workgroups lose up to 15 %, and every workgroup of the abs-max ends in an atomic)
+constexpr long long kCacheBytes = 256ll << 20;  // beyond the last-level cache, streams bypass it (non-temporal): +18 %
+                                                // at 1 GiB, -8 % at 128 MiB, hence the switch
+
+__global__ void zero_float_kernel(float* p) { *p = 0.f; }
+
+// inc/utils.hpp:31-39.  |x| of non-NaN floats orders like its bit pattern, so the grid-wide maximum is an unsigned
+// atomic max on *out, which zero_float_kernel has cleared.
+__global__ __launch_bounds__(kQuantThreads) void abs_max_kernel(const float* __restrict__ x, long long n,
+                                                                 float* __restrict__ out) {
+  const long long units = n / 4;
+  const float4* __restrict__ x4 = reinterpret_cast<const float4*>(x);
+  const long long stride = (long long)gridDim.x * kQuantThreads;
+  float m = 0.f;
+  auto take = [&](float v) {
+    const float a = fabsf(v);
+    m = a > m ? a : m;  // a NaN never compares greater: skipped, as in the reference
+  };
+  // (one running maximum: 16 compare-selects per 64 bytes are far below what the loads cost)
+  long long j = (long long)blockIdx.x * kQuantThreads + threadIdx.x;
+  for (; j + (kQuantUnroll - 1) * stride < units; j += kQuantUnroll * stride) {
+    float4 v[kQuantUnroll];
+#pragma unroll
+    for (int u = 0; u < kQuantUnroll; ++u) v[u] = x4[j + u * stride];
+#pragma unroll
+    for (int u = 0; u < kQuantUnroll; ++u) { take(v[u].x); take(v[u].y); take(v[u].z); take(v[u].w); }
+  }
+  for (; j < units; j += stride) {
+    const float4 v = x4[j];
+    take(v.x); take(v.y); take(v.z); take(v.w);
+  }
+  if (blockIdx.x == 0 && threadIdx.x < (int)(n - 4 * units)) take(x[4 * units + threadIdx.x]);
+  // wavefront, then workgroup, then grid
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float o = __shfl_xor(m, off);
+    m = o > m ? o : m;
+  }
+  __shared__ float part[kQuantThreads / 64];
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int w = 1; w < kQuantThreads / 64; ++w) m = part[w] > m ? part[w] : m;
+    if (m > 0.f) atomicMax(reinterpret_cast<unsigned int*>(out), __float_as_uint(m));
+  }
+}
+
+// inc/utils.hpp:23-29: floorf(x * (127 / amax) + 0.5) in float arithmetic (the reference's double add is exact and
+// floorf takes a float, which is one correctly rounded float add), clamp to [-127, 127]; NaN -> 0.
+__device__ __forceinline__ int quant1(float x, float scale) {
+  const float q = floorf(x * scale + 0.5f);
+  return (int)fminf(fmaxf(q, -127.f), 127.f);  // clamped as a float, so that an infinite product is +-127 too
+}
+__device__ __forceinline__ int quant1_nan0(float x, float scale) {
+  const float p = x * scale;
+  return p == p ? quant1(x, scale) : 0;
+}
+
+template <bool NT>
+__global__ __launch_bounds__(kQuantThreads) void quantize_i8_kernel(const float* __restrict__ x, long long n,
+                                                                     float amax_host,
+                                                                     const float* __restrict__ amax_dev,
+                                                                     int8_t* __restrict__ out) {
+  const float amax = amax_dev != nullptr ? *amax_dev : amax_host;
+  const float scale = 127.0f / amax;
+  const long long units = n / 4;
+  const v4f* __restrict__ x4 = reinterpret_cast<const v4f*>(x);
+  int* __restrict__ o4 = reinterpret_cast<int*>(out);
+  const long long stride = (long long)gridDim.x * kQuantThreads;
+  auto pack = [&](const v4f& v) {
+    return (quant1_nan0(v.x, scale) & 0xff) | ((quant1_nan0(v.y, scale) & 0xff) << 8) |
+           ((quant1_nan0(v.z, scale) & 0xff) << 16) | (quant1_nan0(v.w, scale) << 24);
+  };
+  long long j = (long long)blockIdx.x * kQuantThreads + threadIdx.x;
+  for (; j + (kQuantUnroll - 1) * stride < units; j += kQuantUnroll * stride) {
+    v4f v[kQuantUnroll];
+#pragma unroll
+    for (int u = 0; u < kQuantUnroll; ++u) v[u] = NT ? __builtin_nontemporal_load(&x4[j + u * stride]) : x4[j + u * stride];
+#pragma unroll
+    for (int u = 0; u < kQuantUnroll; ++u) {
+      if (NT) __builtin_nontemporal_store(pack(v[u]), &o4[j + u * stride]);
+      else o4[j + u * stride] = pack(v[u]);
+    }
+  }
+  for (; j < units; j += stride) o4[j] = pack(x4[j]);
+  if (blockIdx.x == 0 && threadIdx.x < (int)(n - 4 * units))
+    out[4 * units + threadIdx.x] = (int8_t)quant1_nan0(x[4 * units + threadIdx.x], scale);
+}
+
+// inc/utils.hpp:53: (float)v / 127.0f * amax, in that order.
+template <bool NT>
+__global__ __launch_bounds__(kQuantThreads) void dequantize_i8_kernel(const int8_t* __restrict__ x, long long n,
+                                                                       float amax, float* __restrict__ out) {
+  const long long units = n / 4;
+  const int* __restrict__ x4 = reinterpret_cast<const int*>(x);
+  v4f* __restrict__ o4 = reinterpret_cast<v4f*>(out);
+  const long long stride = (long long)gridDim.x * kQuantThreads;
+  auto one = [&](int v) { return (float)v / 127.0f * amax; };
+  auto unpack = [&](int w) {
+    return v4f{one((int8_t)(w & 0xff)), one((int8_t)((w >> 8) & 0xff)), one((int8_t)((w >> 16) & 0xff)), one(w >> 24)};
+  };
+  long long j = (long long)blockIdx.x * kQuantThreads + threadIdx.x;
+  for (; j + (kQuantUnroll - 1) * stride < units; j += kQuantUnroll * stride) {
+    int w[kQuantUnroll];
+#pragma unroll
+    for (int u = 0; u < kQuantUnroll; ++u) w[u] = NT ? __builtin_nontemporal_load(&x4[j + u * stride]) : x4[j + u * stride];
+#pragma unroll
+    for (int u = 0; u < kQuantUnroll; ++u) {
+      if (NT) __builtin_nontemporal_store(unpack(w[u]), &o4[j + u * stride]);
+      else o4[j + u * stride] = unpack(w[u]);
+    }
+  }
+  for (; j < units; j += stride) o4[j] = unpack(x4[j]);
+  if (blockIdx.x == 0 && threadIdx.x < (int)(n - 4 * units)) out[4 * units + threadIdx.x] = one(x[4 * units + threadIdx.x]);
+}
+
+inline int quant_blocks(long long n) {
+  const long long want = (n / 4 + (long long)kQuantThreads * kQuantUnroll - 1) / ((long long)kQuantThreads * kQuantUnroll);
+  return (int)(want < 1 ? 1 : (want > kQuantMaxBlocks ? kQuantMaxBlocks : want));
+}
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+inline int launch_status() {
+  const hipError_t err = hipGetLastError();
+  return err == hipSuccess ? FMHA_I8_OK : FMHA_I8_ERR_HIP_BASE + (int)err;
+}
+
+}  // namespace fmha_i8_gfx950
+
+extern "C" {
+
+int FMHAAbsMaxF32(hipStream_t stream, const float* x, long long n, float* amax_out) {
+  using namespace fmha_i8_gfx950;
+  if (amax_out == nullptr || (x == nullptr && n > 0) || n < 0) return FMHA_I8_ERR_NULL_POINTER;
+  if (!aligned16(x)) return FMHA_I8_ERR_ALIGNMENT;
+  hipLaunchKernelGGL(zero_float_kernel, dim3(1), dim3(1), 0, stream, amax_out);
+  if (n > 0) hipLaunchKernelGGL(abs_max_kernel, dim3(quant_blocks(n)), dim3(kQuantThreads), 0, stream, x, n, amax_out);
+  return launch_status();
+}
+
+int FMHAQuantizeI8(hipStream_t stream, const float* x, long long n, float amax_host, const float* amax_dev, int8_t* out) {
+  using namespace fmha_i8_gfx950;
+  if (n < 0 || ((x == nullptr || out == nullptr) && n > 0)) return FMHA_I8_ERR_NULL_POINTER;
+  if (!aligned16(x) || !aligned16(out)) return FMHA_I8_ERR_ALIGNMENT;
+  if (amax_dev == nullptr && !(amax_host == amax_host)) return FMHA_I8_ERR_SCALE;
+  if (n == 0) return FMHA_I8_OK;
+  if (5 * n > kCacheBytes)
+    hipLaunchKernelGGL(quantize_i8_kernel<true>, dim3(quant_blocks(n)), dim3(kQuantThreads), 0, stream, x, n, amax_host,
+                       amax_dev, out);
+  else
+    hipLaunchKernelGGL(quantize_i8_kernel<false>, dim3(quant_blocks(n)), dim3(kQuantThreads), 0, stream, x, n, amax_host,
+                       amax_dev, out);
+  return launch_status();
+}
+
+int FMHADequantizeI8(hipStream_t stream, const int8_t* x, long long n, float amax, float* out) {
+  using namespace fmha_i8_gfx950;
+  if (n < 0 || ((x == nullptr || out == nullptr) && n > 0)) return FMHA_I8_ERR_NULL_POINTER;
+  if (!aligned16(x) || !aligned16(out)) return FMHA_I8_ERR_ALIGNMENT;
+  if (n == 0) return FMHA_I8_OK;
+  if (5 * n > kCacheBytes)
+    hipLaunchKernelGGL(dequantize_i8_kernel<true>, dim3(quant_blocks(n)), dim3(kQuantThreads), 0, stream, x, n, amax, out);
+  else
+    hipLaunchKernelGGL(dequantize_i8_kernel<false>, dim3(quant_blocks(n)), dim3(kQuantThreads), 0, stream, x, n, amax, out);
+  return launch_status();
+}
+
+}  // extern "C"

@@ -85,12 +85,13 @@ void cpu_attention_masked_softmax(const Data* s, Data* p, const int* mask, int b
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// inc/utils.hpp:23-29: scale = 127/amax, floor(x*scale + 0.5) (the 0.5 is a double literal there, so the add and
-// the floor happen in double), clamp to [-127, 127].
+// inc/utils.hpp:23-29: scale = 127/amax, floorf(x*scale + 0.5), clamp to [-127, 127].  The 0.5 is a double literal
+// there, so the add is exact in double, and floorf takes a float, so the sum is rounded to float before the floor: the
+// one float just below 0.5 (0x3EFFFFFF) sums to 1 - 2^-25, rounds to 1.0f and quantises to 1, not 0.
 inline int32_t quantize_i8(float x, float amax) {
   const float scale = 127.0f / amax;
   const float scaled = x * scale;
-  int32_t q = static_cast<int32_t>(std::floor(static_cast<double>(scaled) + 0.5));
+  int32_t q = static_cast<int32_t>(floorf(static_cast<float>(static_cast<double>(scaled) + 0.5)));
   return q < -127 ? -127 : (q > 127 ? 127 : q);
 }
 

@@ -18,10 +18,10 @@ CONFIGS = {
 
 
 def quantize_i8_np(x, amax):
-    """inc/utils.hpp:23-29 in numpy: floor(x * (127/amax) + 0.5) with the add in double, clamp +-127."""
+    """inc/utils.hpp:23-29 in numpy: floorf(x * (127/amax) + 0.5): the add in double, rounded to float for floorf."""
     scale = np.float32(127.0) / np.float32(amax)
     scaled = (x.astype(np.float32) * scale).astype(np.float32)
-    q = np.floor(scaled.astype(np.float64) + 0.5)
+    q = np.floor((scaled.astype(np.float64) + 0.5).astype(np.float32))
     return np.clip(q, -127, 127).astype(np.int8)
 
 

@@ -9,6 +9,8 @@
 //                                           uniform(+-0.5) Q/K, |uniform| V, scattered 20 % mask, o_amax measured
 //   test_fmha_i8 --B 2 --H 4 --S 512 --d 64 [--valid L] [--dist normal|student_t|reference]
 //   common: --seed N --iters N --warmup N --cpu-heads N (0 = all) --cpu-threads N --json FILE --no-check
+//   --quant MiB            instead of attention cases: abs-max, quantise and de-quantise (include/fmha_quant.h) over that
+//                          many MiB of fp32 input, checked bit for bit against the CPU checker and timed against HBM
 //   --calibrate-copy MiB   also run one device-to-device copy of that size, so that a counter run (FETCH_SIZE /
 //                          WRITE_SIZE) sees a plain copy kernel of known traffic to scale the attention kernel's by
 #include <hip/hip_runtime_api.h>
@@ -22,6 +24,7 @@
 #include <vector>
 
 #include "fmha_i8.h"
+#include "fmha_quant.h"
 #include "fmha_oracle.hpp"
 
 inline void check_hip(hipError_t e, const char* file, int line) {
@@ -263,12 +266,69 @@ bool run_case(const Case& c, const Options& opt, FILE* json) {
 
 }  // namespace
 
+// Quantisation front end / back end (include/fmha_quant.h): parity with inc/utils.hpp:23-39,53 and HBM throughput.
+static bool run_quant(long mib, const Options& opt) {
+  const long long n = ((long long)mib << 20) / 4 + 3;  // an element count that is not a multiple of four
+  std::vector<float> x((size_t)n);
+  Rng rng(opt.seed ^ 0x51ull);
+  for (long long i = 0; i < n; ++i) x[(size_t)i] = (float)(3.0 * rng.normal());
+  x[(size_t)(n / 3)] = -17.25f;  // the maximum, a negative number
+  float *dx, *dam, *dback;
+  int8_t* dq;
+  CHECK_HIP(hipMalloc(&dx, (size_t)n * 4)), CHECK_HIP(hipMalloc(&dback, (size_t)n * 4 + 16));
+  CHECK_HIP(hipMalloc(&dq, (size_t)n + 16)), CHECK_HIP(hipMalloc(&dam, 4));
+  CHECK_HIP(hipMemcpy(dx, x.data(), (size_t)n * 4, hipMemcpyHostToDevice));
+  hipStream_t stream;
+  CHECK_HIP(hipStreamCreate(&stream));
+  hipEvent_t e0, e1;
+  CHECK_HIP(hipEventCreate(&e0)), CHECK_HIP(hipEventCreate(&e1));
+  const int iters = opt.iters < 200 ? opt.iters : 200, warm = opt.warmup < 50 ? opt.warmup : 50;
+  auto timed = [&](const char* what, double bytes, auto&& call) {
+    for (int i = 0; i < warm; ++i) call();
+    CHECK_HIP(hipStreamSynchronize(stream));
+    CHECK_HIP(hipEventRecord(e0, stream));
+    for (int i = 0; i < iters; ++i) call();
+    CHECK_HIP(hipEventRecord(e1, stream));
+    CHECK_HIP(hipEventSynchronize(e1));
+    float ms = 0;
+    CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+    const double us = ms * 1e3 / iters, gbs = bytes / us * 1e-3;
+    printf("%-28s %10.2f us/call  %8.1f GB/s  %5.1f %% of 8000 GB/s HBM peak  (%.0f algorithmic bytes)\n", what, us, gbs,
+           100.0 * gbs / 8000.0, bytes);
+  };
+  int st = 0;
+  timed("FMHAAbsMaxF32", 4.0 * n, [&] { st |= FMHAAbsMaxF32(stream, dx, n, dam); });
+  timed("FMHAQuantizeI8 (device amax)", 5.0 * n, [&] { st |= FMHAQuantizeI8(stream, dx, n, 0.f, dam, dq); });
+  timed("FMHADequantizeI8", 5.0 * n, [&] { st |= FMHADequantizeI8(stream, dq, n, 17.25f, dback); });
+  if (st != FMHA_I8_OK) {
+    fprintf(stderr, "quantisation entry points failed: %s\n", FMHAInferI8StatusString(st));
+    return false;
+  }
+  float amax = 0;
+  std::vector<int8_t> q((size_t)n);
+  std::vector<float> back((size_t)n);
+  CHECK_HIP(hipMemcpy(&amax, dam, 4, hipMemcpyDeviceToHost));
+  CHECK_HIP(hipMemcpy(q.data(), dq, (size_t)n, hipMemcpyDeviceToHost));
+  CHECK_HIP(hipMemcpy(back.data(), dback, (size_t)n * 4, hipMemcpyDeviceToHost));
+  long long bad_q = 0, bad_d = 0;
+  const float want_amax = fmha_oracle::abs_max(x.data(), n);
+  for (long long i = 0; i < n; ++i) {
+    if (q[(size_t)i] != (int8_t)fmha_oracle::quantize_i8(x[(size_t)i], want_amax)) ++bad_q;
+    if (back[(size_t)i] != (float)q[(size_t)i] / 127.0f * 17.25f) ++bad_d;
+  }
+  const bool ok = amax == want_amax && bad_q == 0 && bad_d == 0;
+  printf("quantisation parity over %lld elements: amax %g (checker %g), quantise mismatches %lld, de-quantise mismatches "
+         "%lld  [%s]\n", n, amax, want_amax, bad_q, bad_d, ok ? "PASS" : "FAIL");
+  CHECK_HIP(hipFree(dx)), CHECK_HIP(hipFree(dback)), CHECK_HIP(hipFree(dq)), CHECK_HIP(hipFree(dam));
+  return ok;
+}
+
 int main(int argc, char** argv) {
   Options opt;
   std::vector<Case> cases;
   Case custom;
   bool have_custom = false;
-  long calib_mib = 0;
+  long calib_mib = 0, quant_mib = 0;
   for (int i = 1; i < argc; ++i) {
     const std::string a = argv[i];
     auto val = [&]() -> const char* {
@@ -302,6 +362,7 @@ int main(int argc, char** argv) {
     else if (a == "--no-check") opt.check = false;
     else if (a == "--json") opt.json = val();
     else if (a == "--calibrate-copy") calib_mib = atol(val());
+    else if (a == "--quant") quant_mib = atol(val());
     else {
       fprintf(stderr, "unknown argument %s\n", a.c_str());
       return 2;
@@ -328,6 +389,11 @@ int main(int argc, char** argv) {
     CHECK_HIP(hipDeviceSynchronize());
     CHECK_HIP(hipFree(src)), CHECK_HIP(hipFree(dst));
     printf("calibration copy: %ld MiB device to device (reads %zu bytes, writes %zu bytes)\n", calib_mib, bytes, bytes);
+  }
+  if (quant_mib > 0) {
+    const bool ok = run_quant(quant_mib, opt);
+    printf("%s\n", ok ? "ALL CASES PASS" : "SOME CASES FAILED");
+    return ok ? 0 : 1;
   }
   FILE* json = opt.json.empty() ? nullptr : fopen(opt.json.c_str(), "w");
   bool all = true;

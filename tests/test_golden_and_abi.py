@@ -1,5 +1,5 @@
 """CPU tests: the committed known-answer fixtures still come out of the checker bit for bit, and the C-ABI library
-loads and exports every symbol that include/fmha_i8.h declares (no compute call is made here)."""
+loads and exports every symbol that include/fmha_i8.h and include/fmha_quant.h declare (no compute call is made here)."""
 import ctypes
 import glob
 import os
@@ -26,9 +26,12 @@ def test_checker_reproduces_fixture(orc, path):
 
 
 def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "fmha_i8.h")).read()
-    body = text.split('extern "C" {', 1)[1].split('} /* extern "C" */', 1)[0]
-    return sorted(set(re.findall(r"\b(FMHAInferI8\w*)\s*\(", body)))
+    names = set()
+    for header in ("fmha_i8.h", "fmha_quant.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        body = text.split('extern "C" {', 1)[1].split('} /* extern "C" */', 1)[0]
+        names |= set(re.findall(r"\b(FMHA[A-Z]\w*)\s*\(", body))
+    return sorted(names)
 
 
 def test_library_exports_every_declared_symbol(pkg):

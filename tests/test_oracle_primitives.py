@@ -115,6 +115,11 @@ def test_quantizer_known_answers(orc):
     got = orc.quantize_i8(xs, amax)
     assert np.array_equal(got, want)
     assert np.array_equal(fc.quantize_i8_np(xs, amax), want)
+    # floorf takes a float: with amax = 127 the scale is exactly 1, and the float just below 0.5 rounds up to 1.0f in the
+    # sum and quantises to 1; its neighbour one ulp further down does not
+    edge = np.array([0x3EFFFFFF, 0x3EFFFFFE, 0x3F000000, 0xBF000000, 0xBF000001], np.uint32).view(np.float32)
+    assert np.array_equal(orc.quantize_i8(edge, 127.0), np.array([1, 0, 1, 0, -1], np.int8))
+    assert np.array_equal(fc.quantize_i8_np(edge, 127.0), np.array([1, 0, 1, 0, -1], np.int8))
     rng = np.random.default_rng(5)
     x = rng.standard_normal(10000).astype(np.float32) * 3
     a = orc.abs_max(x)
