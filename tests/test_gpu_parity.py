@@ -281,10 +281,10 @@ def test_cpp_harness_config1_and_reference_sweep(tmp_path):
     exe = os.path.join(HERE, "bin", "test_fmha_i8")
     assert os.path.exists(exe), "tests/bin/test_fmha_i8 is not built (python -c 'import __graft_entry__ as g; g.build()')"
     js = str(tmp_path / "harness.json")
-    r = subprocess.run([exe, "--config", "1", "--sweep", "--iters", "20", "--cpu-heads", "0", "--json", js],
+    r = subprocess.run([exe, "--config", "1", "--sweep", "--iters", "20", "--warmup", "20", "--cpu-heads", "0", "--json", js],
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
     print(r.stdout[-3000:])
     assert r.returncode == 0
     recs = [json.loads(l) for l in open(js)]
-    assert len(recs) == 15 and all(x["pass"] for x in recs)
+    assert len(recs) == 23 and all(x["pass"] for x in recs)
     assert all(x["mean_rel_dev_pct"] < 20.0 for x in recs if x["case"] == "sweep")
