@@ -152,6 +152,40 @@ def test_full_size_properties_c3(pkg, dev):
     del torch
 
 
+@pytest.mark.parametrize("S,d", [(65536, 64), (65472, 64), (16384, 128)])
+def test_longest_sequences_by_closed_forms(pkg, dev, S, d):
+    """The longest sequences the library takes (512 key blocks of 128, or 1023 of 64): no CPU pass of that size finishes
+    in seconds, so the checks are closed forms.  Q == 0 makes attention uniform over the unmasked keys, so that
+    O = rne(clamp(v_amax/o_amax * mean V)); a one-key "needle" (one K row far closer to every Q row than the rest)
+    makes O the V row of that key; determinism; and a masked tail must equal the sequence cut at the same place."""
+    rng = np.random.default_rng(S + d)
+    valid = S - 3 * 64 - 17  # the masked tail covers whole key blocks and a ragged part of one
+    v = rng.integers(-127, 128, (1, 1, S, d), dtype=np.int8)
+    k = rng.integers(-20, 21, (1, 1, S, d), dtype=np.int8)
+    mask = np.zeros((1, S), np.int8)
+    mask[0, valid:] = 1
+    base = dict(k=k, v=v, mask=mask, q_amax=1.0, k_amax=1.0, v_amax=2.0, o_amax=1.0)
+    # uniform attention over the valid keys
+    got = gpu_run(pkg, dev, dict(base, q=np.zeros((1, 1, S, d), np.int8))).astype(np.int64)
+    y = 2.0 * v[0, 0, :valid].astype(np.float64).mean(axis=0)
+    want = np.broadcast_to(np.clip(np.rint(y), -127, 127), got.shape)
+    assert np.abs(got - want).max() <= 1 and (got == want).mean() > 0.99
+    assert np.array_equal(gpu_run(pkg, dev, dict(base, q=np.zeros((1, 1, S, d), np.int8))).astype(np.int64), got)
+    # a needle: key j0 is the only one that matters (score 127*127*d against at most 127*20*d, scaled up by the amax
+    # product), in a block in the middle of the sequence
+    j0 = (valid // 2) | 1
+    kn = k.copy()
+    kn[0, 0, j0] = 127
+    q = np.full((1, 1, S, d), 127, np.int8)
+    got = gpu_run(pkg, dev, dict(base, q=q, k=kn, q_amax=30.0, k_amax=30.0, v_amax=1.0)).astype(np.int64)
+    assert np.array_equal(got[0, 0], np.broadcast_to(v[0, 0, j0].astype(np.int64), (S, d)))
+    # the same needle behind the mask is invisible: the result is then far from that V row
+    kn2 = k.copy()
+    kn2[0, 0, valid + 5] = 127
+    got2 = gpu_run(pkg, dev, dict(base, q=q, k=kn2, q_amax=30.0, k_amax=30.0, v_amax=1.0)).astype(np.int64)
+    assert not np.array_equal(got2[0, 0, 0], v[0, 0, valid + 5].astype(np.int64))
+
+
 def test_full_size_mask_properties_c4(pkg, dev):
     c = fc.make_config("C4")
     base = gpu_run(pkg, dev, c)
@@ -210,6 +244,18 @@ def test_saturation_and_clamp(pkg, orc, dev):
     want = cpu_run(orc, c, v_amax=4 * c["v_amax"])
     assert (np.abs(want) == 127).mean() > 0.02
     check(gpu_run(pkg, dev, c, v_amax=4 * c["v_amax"]), want, "saturating")
+
+
+@pytest.mark.parametrize("S,d", [(512, 128), (512, 64), (320, 128), (320, 64)])
+@pytest.mark.parametrize("qk_scale,vo_ratio", [(1.0, 1.0), (1.0, 60.0), (40.0, 1.0), (40.0, 60.0)])
+def test_every_kernel_variant(pkg, orc, dev, S, d, qk_scale, vo_ratio):
+    """The library picks one of four arithmetic variants of the kernel from the scales (accumulators read as floats or
+    converted; accumulator offset folded into the running O or not) for each head_dim and softmax block size.  A large
+    q_amax*k_amax forces the converting variant, a large v_amax/o_amax the unfolded one: all sixteen instantiations
+    must meet the same gate."""
+    c = fc.make_inputs(2, 2, S, d, dist="normal", pad="scatter", seed=91)
+    kw = dict(q_amax=c["q_amax"] * qk_scale, v_amax=vo_ratio, o_amax=1.0 if vo_ratio == 1.0 else 2.0)
+    check(gpu_run(pkg, dev, c, **kw), cpu_run(orc, c, **kw), "variant S=%d d=%d qk=%g vo=%g" % (S, d, qk_scale, vo_ratio))
 
 
 def test_masked_sentinel_corner(pkg, orc, dev):
