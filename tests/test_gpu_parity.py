@@ -305,6 +305,41 @@ def test_void_entry_point_streams_and_use_tcu_flag(pkg, orc, dev):
         check(o.cpu().numpy(), want, "void entry use_tcu=%s" % use_tcu)
 
 
+def test_graph_capture_and_replay(pkg, orc, dev):
+    """The call allocates nothing and never synchronises, so it can be recorded into a HIP graph: capture one launch,
+    replay it several times with eager work and synchronisations in between and with new inputs written into the same
+    buffers, and check every replay against the eager result."""
+    import torch
+    c = fc.make_inputs(2, 2, 384, 128, dist="normal", pad="scatter", seed=61)
+    q, k, v, m = to_dev(dev, c["q"], c["k"], c["v"], c["mask"])
+    o = torch.zeros_like(q)
+    P = pkg.FMHAParamI8(c["q_amax"], c["k_amax"], c["v_amax"], c["o_amax"])
+    A = pkg.AttnDataDescriptor(2, 384, 2, 128)
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        assert pkg.FMHAInferI8Status(side, P, A, q, k, v, m, o, True) == 0  # warm-up outside the capture
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        assert pkg.FMHAInferI8Status(torch.cuda.current_stream(dev), P, A, q, k, v, m, o, True) == 0
+    want = cpu_run(orc, c)
+    for rep in range(4):
+        if rep == 2:  # new inputs in the same buffers: the graph holds pointers, not data
+            c = fc.make_inputs(2, 2, 384, 128, dist="normal", pad="scatter", seed=62)
+            for dst, name in ((q, "q"), (k, "k"), (v, "v"), (m, "mask")):
+                dst.copy_(torch.from_numpy(c[name]))
+            want = cpu_run(orc, dict(c, q_amax=P.q_amax, k_amax=P.k_amax, v_amax=P.v_amax, o_amax=P.o_amax))
+        o.fill_(77)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = pkg.fmha_infer_i8(q, k, v, m, P.q_amax, P.k_amax, P.v_amax, P.o_amax)
+        torch.cuda.synchronize()
+        assert torch.equal(o, eager), rep
+        check(o.cpu().numpy(), want, "graph replay %d" % rep)
+
+
 def test_unsupported_shapes_leave_output_untouched(pkg, dev):
     import torch
     q = torch.zeros(1, 1, 160, 64, dtype=torch.int8, device=dev)
