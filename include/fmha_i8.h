@@ -40,7 +40,7 @@ extern "C" {
 #define FMHA_I8_OK 0
 #define FMHA_I8_ERR_NULL_POINTER 1   /* q, k, v, padding_mask or o is NULL */
 #define FMHA_I8_ERR_HEAD_DIM 2       /* head_dim not in {64, 128} */
-#define FMHA_I8_ERR_SEQ_LEN 3        /* seq_len <= 0, not a multiple of 64, or > 65536 */
+#define FMHA_I8_ERR_SEQ_LEN 3        /* key seq_len <= 0, not a multiple of 64, or > 65536; query seq_len <= 0 or > 65536 */
 #define FMHA_I8_ERR_BATCH_HEAD 4     /* batch_num or head_num <= 0, or the grid would exceed HIP limits */
 #define FMHA_I8_ERR_ALIGNMENT 5      /* q, k, v or o not 16-byte aligned */
 #define FMHA_I8_ERR_SCALE 6          /* an amax is not finite, or o_amax <= 0 */
@@ -64,7 +64,31 @@ int FMHAInferI8Status(hipStream_t stream, FMHAParamI8 fmha_param, AttnDataDescri
 int FMHAInferI8CheckArgs(FMHAParamI8 fmha_param, AttnDataDescriptor attn_desc, const void* q, const void* k,
                          const void* v, const void* padding_mask, const void* o);
 
-/* Human-readable text for a status code returned by the two functions above (static storage). */
+/* Shape of a call whose queries and keys differ in number: what the reference lists as planned ("S_src != S_dst",
+ * README.md:13) and its kernel cannot express (one SEQ_LEN template parameter sizes Q, K, V and the mask alike,
+ * inc/fmha_i8.cuh:45,88-89). */
+typedef struct FMHACrossAttnDescriptor {
+  int batch_num;
+  int seq_len_q;   /* rows of q and o per head: any count from 1 to 65536 */
+  int seq_len_kv;  /* rows of k and v per head, and mask bytes per batch entry: a positive multiple of 64, <= 65536 */
+  int head_num;
+  int head_dim;
+} FMHACrossAttnDescriptor;
+
+/* Attention of seq_len_q queries over seq_len_kv keys.  q, o: int8 [batch_num, head_num, seq_len_q, head_dim];
+ * k, v: int8 [batch_num, head_num, seq_len_kv, head_dim]; padding_mask: int8 [batch_num, seq_len_kv].  Everything
+ * else (scales, numerics, ownership, asynchrony, status codes) as for FMHAInferI8Status; the softmax block is 128 keys
+ * when seq_len_kv is a multiple of 128, else 64.  Query rows are independent of each other, so with
+ * seq_len_q == seq_len_kv this IS FMHAInferI8Status (same kernel, same launch), and a call on the first n query rows
+ * of a self-attention problem gives the first n rows of its output. */
+int FMHAInferI8Cross(hipStream_t stream, FMHAParamI8 fmha_param, FMHACrossAttnDescriptor desc, const void* q,
+                     const void* k, const void* v, const void* padding_mask, void* o);
+
+/* Argument check only, no HIP call: what FMHAInferI8Cross would return before launching. */
+int FMHAInferI8CrossCheckArgs(FMHAParamI8 fmha_param, FMHACrossAttnDescriptor desc, const void* q, const void* k,
+                              const void* v, const void* padding_mask, const void* o);
+
+/* Human-readable text for a status code returned by the functions above (static storage). */
 const char* FMHAInferI8StatusString(int status);
 
 /* Library build identification: "fmha_i8 gfx950 <variant>" (static storage). */

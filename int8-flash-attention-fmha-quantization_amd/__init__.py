@@ -16,7 +16,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libfmha_i8.so")
 
 EXPORTED_SYMBOLS = ("FMHAInferI8", "FMHAInferI8Status", "FMHAInferI8CheckArgs", "FMHAInferI8StatusString",
-                    "FMHAInferI8Version", "FMHAAbsMaxF32", "FMHAQuantizeI8", "FMHADequantizeI8")
+                    "FMHAInferI8Version", "FMHAInferI8Cross", "FMHAInferI8CrossCheckArgs", "FMHAAbsMaxF32",
+                    "FMHAQuantizeI8", "FMHADequantizeI8")
 
 FMHA_I8_OK = 0
 FMHA_I8_ERR_NULL_POINTER = 1
@@ -34,6 +35,12 @@ class AttnDataDescriptor(C.Structure):
 
     def __init__(self, batch_num=1, seq_len=64, head_num=4, head_dim=64):
         super().__init__(batch_num, seq_len, head_num, head_dim)
+
+
+class FMHACrossAttnDescriptor(C.Structure):
+    """include/fmha_i8.h: queries and keys differ in number (README.md:13 lists "S_src != S_dst" as planned)."""
+    _fields_ = [("batch_num", C.c_int), ("seq_len_q", C.c_int), ("seq_len_kv", C.c_int), ("head_num", C.c_int),
+                ("head_dim", C.c_int)]
 
 
 class FMHAParamI8(C.Structure):
@@ -83,6 +90,10 @@ def load_library(path=None):
     L.FMHAInferI8StatusString.restype = C.c_char_p
     L.FMHAInferI8Version.argtypes = []
     L.FMHAInferI8Version.restype = C.c_char_p
+    L.FMHAInferI8Cross.argtypes = [ptr, FMHAParamI8, FMHACrossAttnDescriptor, ptr, ptr, ptr, ptr, ptr]
+    L.FMHAInferI8Cross.restype = C.c_int
+    L.FMHAInferI8CrossCheckArgs.argtypes = [FMHAParamI8, FMHACrossAttnDescriptor, ptr, ptr, ptr, ptr, ptr]
+    L.FMHAInferI8CrossCheckArgs.restype = C.c_int
     # include/fmha_quant.h
     L.FMHAAbsMaxF32.argtypes = [ptr, ptr, C.c_longlong, ptr]
     L.FMHAAbsMaxF32.restype = C.c_int
@@ -126,6 +137,17 @@ def FMHAInferI8Status(stream, fmha_param, attn_desc, q, k, v, padding_mask, o, u
 def FMHAInferI8CheckArgs(fmha_param, attn_desc, q, k, v, padding_mask, o):
     return int(load_library().FMHAInferI8CheckArgs(fmha_param, attn_desc, _ptr(q), _ptr(k), _ptr(v),
                                                    _ptr(padding_mask), _ptr(o)))
+
+
+def FMHAInferI8Cross(stream, fmha_param, desc, q, k, v, padding_mask, o):
+    """seq_len_q queries over seq_len_kv keys; status code of include/fmha_i8.h."""
+    return int(load_library().FMHAInferI8Cross(_stream(stream), fmha_param, desc, _ptr(q), _ptr(k), _ptr(v),
+                                               _ptr(padding_mask), _ptr(o)))
+
+
+def FMHAInferI8CrossCheckArgs(fmha_param, desc, q, k, v, padding_mask, o):
+    return int(load_library().FMHAInferI8CrossCheckArgs(fmha_param, desc, _ptr(q), _ptr(k), _ptr(v),
+                                                        _ptr(padding_mask), _ptr(o)))
 
 
 def status_string(status):
@@ -188,22 +210,29 @@ def dequantize_tensor(x, amax, stream=None):
 def fmha_infer_i8(q, k, v, padding_mask, q_amax, k_amax, v_amax, o_amax=1.0, out=None, stream=None):
     """Convenience over FMHAInferI8Status for torch int8 tensors on the GPU.
 
-    q, k, v: int8 [B, H, S, d] contiguous; padding_mask: int8 [B, S], nonzero = key masked out
-    (inc/fmha_i8.cuh:189-192).  Returns int8 O [B, H, S, d].  Raises FMHAError on a nonzero status."""
+    q: int8 [B, H, Sq, d]; k, v: int8 [B, H, S, d], all contiguous; padding_mask: int8 [B, S], nonzero = key masked
+    out (inc/fmha_i8.cuh:189-192).  Returns int8 O [B, H, Sq, d].  Sq == S goes through the reference's entry point
+    (FMHAInferI8Status), anything else through FMHAInferI8Cross.  Raises FMHAError on a nonzero status."""
     import torch
 
     for name, t in (("q", q), ("k", k), ("v", v), ("padding_mask", padding_mask)):
         if not (t.is_cuda and t.dtype == torch.int8 and t.is_contiguous()):
             raise ValueError("%s must be a contiguous int8 tensor on the GPU" % name)
-    B, H, S, d = q.shape
-    if k.shape != q.shape or v.shape != q.shape or tuple(padding_mask.shape) != (B, S):
-        raise ValueError("shape mismatch: q/k/v [B,H,S,d] and padding_mask [B,S] expected")
+    B, H, Sq, d = q.shape
+    S = k.shape[2] if k.dim() == 4 else -1
+    if tuple(k.shape) != (B, H, S, d) or v.shape != k.shape or tuple(padding_mask.shape) != (B, S):
+        raise ValueError("shape mismatch: q [B,H,Sq,d], k/v [B,H,S,d] and padding_mask [B,S] expected")
     if out is None:
         out = torch.empty_like(q)
+    elif not (out.is_cuda and out.dtype == torch.int8 and out.is_contiguous() and out.shape == q.shape):
+        raise ValueError("out must be a contiguous int8 tensor on the GPU, shaped like q")
     if stream is None:
         stream = torch.cuda.current_stream(q.device)
-    st = FMHAInferI8Status(stream, FMHAParamI8(q_amax, k_amax, v_amax, o_amax, 1.0), AttnDataDescriptor(B, S, H, d),
-                           q, k, v, padding_mask, out, True)
+    param = FMHAParamI8(q_amax, k_amax, v_amax, o_amax, 1.0)
+    if Sq == S:
+        st = FMHAInferI8Status(stream, param, AttnDataDescriptor(B, S, H, d), q, k, v, padding_mask, out, True)
+    else:
+        st = FMHAInferI8Cross(stream, param, FMHACrossAttnDescriptor(B, Sq, S, H, d), q, k, v, padding_mask, out)
     if st != FMHA_I8_OK:
         raise FMHAError(st, status_string(st))
     return out

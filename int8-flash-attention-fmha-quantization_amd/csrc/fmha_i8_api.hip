@@ -13,14 +13,20 @@ namespace {
 
 using fmha_i8_gfx950::KernelArgs;
 
-int check_args(const FMHAParamI8& p, const AttnDataDescriptor& a, const void* q, const void* k, const void* v,
+// One shape for both entry points: self-attention is the case seq_len_q == seq_len_kv.
+FMHACrossAttnDescriptor as_cross(const AttnDataDescriptor& a) {
+  return FMHACrossAttnDescriptor{a.batch_num, a.seq_len, a.seq_len, a.head_num, a.head_dim};
+}
+
+int check_args(const FMHAParamI8& p, const FMHACrossAttnDescriptor& a, const void* q, const void* k, const void* v,
                const void* mask, const void* o) {
   if (!q || !k || !v || !mask || !o) return FMHA_I8_ERR_NULL_POINTER;
   if (a.head_dim != 64 && a.head_dim != 128) return FMHA_I8_ERR_HEAD_DIM;
-  if (a.seq_len <= 0 || a.seq_len % fmha_i8_gfx950::kBlockKSmall != 0 || a.seq_len > 65536)
+  if (a.seq_len_kv <= 0 || a.seq_len_kv % fmha_i8_gfx950::kBlockKSmall != 0 || a.seq_len_kv > 65536)
     return FMHA_I8_ERR_SEQ_LEN;
+  if (a.seq_len_q <= 0 || a.seq_len_q > 65536) return FMHA_I8_ERR_SEQ_LEN;
   if (a.batch_num <= 0 || a.head_num <= 0) return FMHA_I8_ERR_BATCH_HEAD;
-  const long long wgs = (long long)a.batch_num * a.head_num * ((a.seq_len + fmha_i8_gfx950::kBlockQ - 1) / fmha_i8_gfx950::kBlockQ);
+  const long long wgs = (long long)a.batch_num * a.head_num * ((a.seq_len_q + fmha_i8_gfx950::kBlockQ - 1) / fmha_i8_gfx950::kBlockQ);
   if (wgs > 0x7fffffffLL) return FMHA_I8_ERR_BATCH_HEAD;
   const uintptr_t bits = (uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o;
   if (bits & 15u) return FMHA_I8_ERR_ALIGNMENT;
@@ -38,7 +44,7 @@ void launch_variant(bool bias, bool fast, dim3 grid, dim3 block, hipStream_t str
 #undef FMHA_LAUNCH
 }
 
-int launch(hipStream_t stream, const FMHAParamI8& p, const AttnDataDescriptor& a, const void* q, const void* k,
+int launch(hipStream_t stream, const FMHAParamI8& p, const FMHACrossAttnDescriptor& a, const void* q, const void* k,
            const void* v, const void* mask, void* o) {
   const int st = check_args(p, a, q, k, v, mask, o);
   if (st != FMHA_I8_OK) return st;
@@ -49,9 +55,10 @@ int launch(hipStream_t stream, const FMHAParamI8& p, const AttnDataDescriptor& a
   args.v = static_cast<const int8_t*>(v);
   args.mask = static_cast<const int8_t*>(mask);
   args.o = static_cast<int8_t*>(o);
-  args.seq_len = a.seq_len;
+  args.seq_q = a.seq_len_q;
+  args.seq_kv = a.seq_len_kv;
   args.head_num = a.head_num;
-  args.q_blocks = (a.seq_len + fmha_i8_gfx950::kBlockQ - 1) / fmha_i8_gfx950::kBlockQ;
+  args.q_blocks = (a.seq_len_q + fmha_i8_gfx950::kBlockQ - 1) / fmha_i8_gfx950::kBlockQ;
   args.total_wgs = a.batch_num * a.head_num * args.q_blocks;
   // inc/fmha_i8.cuh:71-72: row_scale = 1/sqrt(d), scale_qk_out = q_amax*k_amax/127^2; folded with log2(e).
   const float row_scale = 1.0f / sqrtf((float)a.head_dim);
@@ -71,8 +78,8 @@ int launch(hipStream_t stream, const FMHAParamI8& p, const AttnDataDescriptor& a
   // LSBs that is at most about 0.0034 * (v_amax/o_amax) * sqrt(key blocks).  Take it while that stays below 0.1 LSB.
   // Blocks of 128 keys, as the reference uses for its multiples of 128; its other lengths (64, 192, 320, 448:
   // src/fmha_i8.cu:41-60) run in blocks of 64 keys, and so does every other odd multiple of 64 here.
-  const int block_keys = a.seq_len % fmha_i8_gfx950::kBlockK == 0 ? fmha_i8_gfx950::kBlockK : fmha_i8_gfx950::kBlockKSmall;
-  const float lsb_bound = 0.0034f * fabsf(p.v_amax / p.o_amax) * sqrtf((float)(a.seq_len / block_keys));
+  const int block_keys = a.seq_len_kv % fmha_i8_gfx950::kBlockK == 0 ? fmha_i8_gfx950::kBlockK : fmha_i8_gfx950::kBlockKSmall;
+  const float lsb_bound = 0.0034f * fabsf(p.v_amax / p.o_amax) * sqrtf((float)(a.seq_len_kv / block_keys));
   const bool fast = lsb_bound < 0.1f;
   if (a.head_dim == 128) {
     if (block_keys == fmha_i8_gfx950::kBlockK) launch_variant<128, fmha_i8_gfx950::kBlockK>(bias, fast, grid, block, stream, args);
@@ -91,17 +98,27 @@ extern "C" {
 
 int FMHAInferI8CheckArgs(FMHAParamI8 fmha_param, AttnDataDescriptor attn_desc, const void* q, const void* k,
                          const void* v, const void* padding_mask, const void* o) {
-  return check_args(fmha_param, attn_desc, q, k, v, padding_mask, o);
+  return check_args(fmha_param, as_cross(attn_desc), q, k, v, padding_mask, o);
 }
 
 int FMHAInferI8Status(hipStream_t stream, FMHAParamI8 fmha_param, AttnDataDescriptor attn_desc, const void* q,
                       const void* k, const void* v, const void* padding_mask, void* o, bool /*use_tcu*/) {
-  return launch(stream, fmha_param, attn_desc, q, k, v, padding_mask, o);
+  return launch(stream, fmha_param, as_cross(attn_desc), q, k, v, padding_mask, o);
+}
+
+int FMHAInferI8Cross(hipStream_t stream, FMHAParamI8 fmha_param, FMHACrossAttnDescriptor desc, const void* q,
+                     const void* k, const void* v, const void* padding_mask, void* o) {
+  return launch(stream, fmha_param, desc, q, k, v, padding_mask, o);
+}
+
+int FMHAInferI8CrossCheckArgs(FMHAParamI8 fmha_param, FMHACrossAttnDescriptor desc, const void* q, const void* k,
+                              const void* v, const void* padding_mask, const void* o) {
+  return check_args(fmha_param, desc, q, k, v, padding_mask, o);
 }
 
 void FMHAInferI8(hipStream_t stream, FMHAParamI8 fmha_param, AttnDataDescriptor attn_desc, const void* q, const void* k,
                  const void* v, const void* padding_mask, void* o, bool /*use_tcu*/) {
-  const int st = launch(stream, fmha_param, attn_desc, q, k, v, padding_mask, o);
+  const int st = launch(stream, fmha_param, as_cross(attn_desc), q, k, v, padding_mask, o);
   if (st != FMHA_I8_OK)
     fprintf(stderr, "FMHAInferI8: nothing launched, o left untouched: %s (B=%d H=%d S=%d d=%d)\n",
             FMHAInferI8StatusString(st), attn_desc.batch_num, attn_desc.head_num, attn_desc.seq_len,
@@ -113,7 +130,7 @@ const char* FMHAInferI8StatusString(int status) {
     case FMHA_I8_OK: return "ok";
     case FMHA_I8_ERR_NULL_POINTER: return "null pointer argument";
     case FMHA_I8_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
-    case FMHA_I8_ERR_SEQ_LEN: return "seq_len must be a positive multiple of 64, at most 65536";
+    case FMHA_I8_ERR_SEQ_LEN: return "seq_len (of the keys) must be a positive multiple of 64, at most 65536; of the queries 1 to 65536";
     case FMHA_I8_ERR_BATCH_HEAD: return "batch_num and head_num must be positive (and the grid must fit)";
     case FMHA_I8_ERR_ALIGNMENT: return "q, k, v and o must be 16-byte aligned";
     case FMHA_I8_ERR_SCALE: return "amax values must be finite and o_amax > 0";

@@ -62,9 +62,10 @@ struct KernelArgs {
   const int8_t* v;
   const int8_t* mask;
   int8_t* o;
-  int seq_len;
+  int seq_q;        // query (and output) rows per head: any positive count
+  int seq_kv;       // key/value rows per head and mask bytes per batch entry: a multiple of BK
   int head_num;
-  int q_blocks;     // ceil(seq_len / kBlockQ)
+  int q_blocks;     // ceil(seq_q / kBlockQ)
   int total_wgs;    // batch * head_num * q_blocks
   float c2;         // log2(e) * (1/sqrt(d)) * q_amax*k_amax/127^2 : int32 S -> base-2 exponent
   float floor2;     // log2(e) * -1e6 : the reference's initial block maximum (inc/fmha_i8.cuh:116)
@@ -144,15 +145,17 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   const int bh = wg / args.q_blocks;
   const int qb = wg - bh * args.q_blocks;
   const int b = bh / args.head_num;
-  const int S = args.seq_len;
-  const long head_off = (long)bh * S * D;
+  const int S = args.seq_kv;
+  const int Sq = args.seq_q;
+  const long head_off = (long)bh * S * D;    // of K and V
+  const long q_head_off = (long)bh * Sq * D; // of Q and O
   const int8_t* __restrict__ kg = args.k + head_off;
   const int8_t* __restrict__ vg = args.v + head_off;
   const int8_t* __restrict__ mg = args.mask + (long)b * S;
   const int n_blocks = S / BK;
 
   // The prologue puts every cold miss in flight before it waits for any of them: the mask bytes, the first two K/V
-  // tiles (tile 1 on speculation: it exists whenever seq_len >= 256, whether or not its keys are masked) and the Q rows.
+  // tiles (tile 1 on speculation: it exists whenever seq_kv >= 256, whether or not its keys are masked) and the Q rows.
   // ---- per-lane addressing -----------------------------------------------------------------------------------------
   // direct-to-LDS loads: lane l of a 1 KiB region lands at byte 16*l of the region, so the lane FETCHES the chunk that
   // the swizzle assigns to that slot.
@@ -212,7 +215,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // (the next tiles follow right after the first barrier: the CU's vector memory path moves 64 bytes per cycle, and
   // everything queued here delays the first GEMM.)
   const int row0 = qb * kBlockQ + wave * 32;  // first query row of this wavefront
-  const bool active = row0 < S;               // seq_len is a multiple of 128, not of 256: the last workgroup may be half empty
+  const bool active = row0 < Sq;              // the last workgroup of a head may be partly empty
   int mask_word;
   {
     const int j = 4 * tid < S ? 4 * tid : S - 4;
@@ -221,9 +224,10 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   issue_k(0);
   v4i qreg[kDSteps];  // Q: B operand of GEMM 1, loaded once
   {
-    // wavefronts past the end of the sequence load row 0 (unused) so that every wavefront has the same loads in flight
-    const int8_t* qp = args.q + head_off;
-    const int qoff = ((active ? row0 : 0) + i32) * D + 16 * g;
+    // rows past the end of the sequence load the last row (unused) so that every wavefront has the same loads in flight
+    const int8_t* qp = args.q + q_head_off;
+    const int qrow = row0 + i32 < Sq ? row0 + i32 : Sq - 1;
+    const int qoff = qrow * D + 16 * g;
 #pragma unroll
     for (int kk = 0; kk < kDSteps; ++kk)
       asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(qreg[kk]) : "v"(qoff + 32 * kk), "s"(qp) : "memory");
@@ -602,7 +606,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // Lanes l and l+32 hold the g = 0 / g = 1 words of the same query row.  One v_permlane32_swap per word hands lane l
   // both words of output tile u and lane l+32 both words of tile u+1: every lane then owns 32 contiguous bytes of a
   // row and writes them with two 128-bit stores instead of eight scattered 32-bit ones.
-  int8_t* op = args.o + head_off + (long)(row0 + i32) * D + 32 * g;
+  if (row0 + i32 >= Sq) return;  // (no barrier follows)
+  int8_t* op = args.o + q_head_off + (long)(row0 + i32) * D + 32 * g;
 #pragma unroll
   for (int u = 0; u < kDSteps; u += 2) {
     int g0[4], g1[4];

@@ -148,14 +148,18 @@ inline void parallel_for(long n, int threads, F&& body) {
 
 // ---------------------------------------------------------------------------------------------------------------
 // The int8 pipeline of inc/fmha_i8.cuh for ONE (batch, head), all query rows.
-//   q, k, v, o : int8 [S][d] of this head;  mask: int8 [S] of this batch, nonzero = masked out (fmha_i8.cuh:189-192)
+//   k, v : int8 [S][d] of this head;  mask: int8 [S] of this batch, nonzero = masked out (fmha_i8.cuh:189-192)
+//   q, o : int8 [Sq][d] of this head.  The reference has Sq == S only (one SEQ_LEN sizes everything, fmha_i8.cuh:45);
+//          each query row is processed on its own below, as it is in the reference (a warp's 16 rows share nothing
+//          but the K/V tiles), so any Sq is the same arithmetic applied to another number of rows.
 //   block      : keys per softmax block (BASE_SEQ_LEN: 128, or 64 for the reference's 64-multiples)
 // Differences from the reference kernel, both deliberate and both outside what its own test exercises:
 //   * a key block with every key masked is skipped (reference: harmless when it is not the first block, NaN when it
 //     is, fmha_i8.cuh:91-92,116-117,301-310);
 //   * a row with no unmasked key at all yields 0 (as inc/cpuSoftmax.hpp:18-47 does).
 inline void fmha_i8_head_blockwise(const int8_t* q, const int8_t* k, const int8_t* v, const int8_t* mask, int8_t* o,
-                                   int S, int d, float q_amax, float k_amax, float v_amax, float o_amax, int block) {
+                                   int Sq, int S, int d, float q_amax, float k_amax, float v_amax, float o_amax,
+                                   int block) {
   const float row_scale = reference_row_scale(d);                    // fmha_i8.cuh:71
   const float scale_qk_out = q_amax * k_amax / (127.f * 127.f);      // fmha_i8.cuh:72
   const float scale_v_out = v_amax * (1.0f / (o_amax * 128.f));      // fmha_i8.cuh:318
@@ -165,7 +169,7 @@ inline void fmha_i8_head_blockwise(const int8_t* q, const int8_t* k, const int8_
   std::vector<int32_t> p_i8(block);
   std::vector<int32_t> o_tilde(d);
   std::vector<float> o_f(d);
-  for (int i = 0; i < S; ++i) {
+  for (int i = 0; i < Sq; ++i) {
     float m_old = -1e6f, l_old = 0.0f;                                // fmha_i8.cuh:91-92
     std::fill(o_f.begin(), o_f.end(), 0.0f);                          // fmha_i8.cuh:105-108
     const int8_t* qi = q + (long)i * d;
@@ -225,18 +229,26 @@ inline void fmha_i8_head_blockwise(const int8_t* q, const int8_t* k, const int8_
 }
 
 // All heads in [head_begin, head_end) of the flattened (batch*head_num) index; others are left untouched in `o`.
-inline void fmha_i8_cpu_blockwise(const int8_t* q, const int8_t* k, const int8_t* v, const int8_t* mask, int8_t* o,
-                                  int B, int H, int S, int d, float q_amax, float k_amax, float v_amax, float o_amax,
-                                  int block, int threads, long head_begin, long head_end) {
-  const long hd = (long)S * d;
+// q, o: [B][H][Sq][d]; k, v: [B][H][S][d]; mask: [B][S].
+inline void fmha_i8_cpu_blockwise_cross(const int8_t* q, const int8_t* k, const int8_t* v, const int8_t* mask,
+                                        int8_t* o, int B, int H, int Sq, int S, int d, float q_amax, float k_amax,
+                                        float v_amax, float o_amax, int block, int threads, long head_begin,
+                                        long head_end) {
+  const long hd_q = (long)Sq * d, hd = (long)S * d;
   head_begin = std::max<long>(head_begin, 0);
   head_end = std::min<long>(head_end, (long)B * H);
   parallel_for(head_end - head_begin, threads, [&](long t) {
     const long bh = head_begin + t;
     const long b = bh / H;
-    fmha_i8_head_blockwise(q + bh * hd, k + bh * hd, v + bh * hd, mask + b * S, o + bh * hd, S, d, q_amax, k_amax,
-                           v_amax, o_amax, block);
+    fmha_i8_head_blockwise(q + bh * hd_q, k + bh * hd, v + bh * hd, mask + b * S, o + bh * hd_q, Sq, S, d, q_amax,
+                           k_amax, v_amax, o_amax, block);
   });
+}
+inline void fmha_i8_cpu_blockwise(const int8_t* q, const int8_t* k, const int8_t* v, const int8_t* mask, int8_t* o,
+                                  int B, int H, int S, int d, float q_amax, float k_amax, float v_amax, float o_amax,
+                                  int block, int threads, long head_begin, long head_end) {
+  fmha_i8_cpu_blockwise_cross(q, k, v, mask, o, B, H, S, S, d, q_amax, k_amax, v_amax, o_amax, block, threads,
+                              head_begin, head_end);
 }
 
 // ---------------------------------------------------------------------------------------------------------------

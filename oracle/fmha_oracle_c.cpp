@@ -40,6 +40,13 @@ void oracle_fmha_i8_blockwise(const int8_t* q, const int8_t* k, const int8_t* v,
   fmha_i8_cpu_blockwise(q, k, v, mask, o, B, H, S, d, q_amax, k_amax, v_amax, o_amax, block, threads, head_begin,
                         head_end);
 }
+// The same pipeline with Sq query rows over S keys (README.md:13 lists it as planned; the rows are independent).
+void oracle_fmha_i8_blockwise_cross(const int8_t* q, const int8_t* k, const int8_t* v, const int8_t* mask, int8_t* o,
+                                    int B, int H, int Sq, int S, int d, float q_amax, float k_amax, float v_amax,
+                                    float o_amax, int block, int threads, long head_begin, long head_end) {
+  fmha_i8_cpu_blockwise_cross(q, k, v, mask, o, B, H, Sq, S, d, q_amax, k_amax, v_amax, o_amax, block, threads,
+                              head_begin, head_end);
+}
 // test_fmha_i8.cpp:141-162 float path.
 void oracle_fmha_fp32(const float* q, const float* k, const float* v, const int8_t* mask, float* o, int B, int H, int S,
                       int d, int threads, long head_begin, long head_end) {

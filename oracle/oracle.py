@@ -51,6 +51,10 @@ def lib():
         L.oracle_fmha_i8_blockwise.argtypes = [_i8p, _i8p, _i8p, _i8p, _i8p, C.c_int, C.c_int, C.c_int, C.c_int,
                                                C.c_float, C.c_float, C.c_float, C.c_float, C.c_int, C.c_int, C.c_long,
                                                C.c_long]
+        L.oracle_fmha_i8_blockwise_cross.argtypes = [_i8p, _i8p, _i8p, _i8p, _i8p, C.c_int, C.c_int, C.c_int, C.c_int,
+                                                     C.c_int, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int,
+                                                     C.c_int, C.c_long, C.c_long]
+        L.oracle_fmha_i8_blockwise_cross.restype = None
         L.oracle_fmha_fp32.argtypes = [_f32p, _f32p, _f32p, _i8p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
                                        C.c_long, C.c_long]
         L.oracle_hardware_threads.restype = C.c_int
@@ -139,6 +143,22 @@ def fmha_i8_blockwise(q, k, v, mask, q_amax, k_amax, v_amax, o_amax, block=128, 
     lib().oracle_fmha_i8_blockwise(q.reshape(-1), k.reshape(-1), v.reshape(-1), mask.reshape(-1), o.reshape(-1), B, H,
                                    S, d, q_amax, k_amax, v_amax, o_amax, block,
                                    threads or hardware_threads(), hb, he)
+    return o
+
+
+def fmha_i8_blockwise_cross(q, k, v, mask, q_amax, k_amax, v_amax, o_amax, block=None, threads=None):
+    """q: int8 [B,H,Sq,d]; k, v: int8 [B,H,S,d]; mask: int8 [B,S], nonzero = masked out.  Returns int8 O [B,H,Sq,d].
+    block defaults to what the reference's ladder would give S: 128 keys for multiples of 128, else 64."""
+    B, H, Sq, d = q.shape
+    S = k.shape[2]
+    q, k, v = (np.ascontiguousarray(t, dtype=np.int8) for t in (q, k, v))
+    mask = np.ascontiguousarray(mask, dtype=np.int8)
+    assert k.shape == (B, H, S, d) and v.shape == k.shape and mask.shape == (B, S)
+    o = np.zeros_like(q)
+    lib().oracle_fmha_i8_blockwise_cross(q.reshape(-1), k.reshape(-1), v.reshape(-1), mask.reshape(-1), o.reshape(-1),
+                                         B, H, Sq, S, d, q_amax, k_amax, v_amax, o_amax,
+                                         block or (128 if S % 128 == 0 else 64), threads or hardware_threads(),
+                                         0, B * H)
     return o
 
 

@@ -1,0 +1,147 @@
+"""Queries and keys that differ in number (the reference lists "S_src != S_dst" as planned, README.md:13; its kernel
+sizes Q, K, V and the mask by one SEQ_LEN, inc/fmha_i8.cuh:45,88-89).  Nothing in the reference computes this case,
+so parity is anchored on what the reference's arithmetic fixes: a query row never sees another query row
+(inc/fmha_i8.cuh:120-332 keeps m, l and O per row), hence attention of any set of query rows over a key set equals the
+same rows of a self-attention problem over that key set.  The CPU tests pin the checker's cross-length entry to its
+self-attention entry (itself pinned by closed forms and the reference's headers); the GPU tests hold the HIP kernel to
+the checker with the usual gate, and to its own self-attention output bit for bit."""
+import numpy as np
+import pytest
+
+import fmha_cases as fc
+
+WITHIN1_MIN = 0.999
+MAX_ABS_LSB = 2
+
+
+def _scales(c):
+    return c["q_amax"], c["k_amax"], c["v_amax"], c["o_amax"]
+
+
+def _self(orc, c):
+    S = c["k"].shape[2]
+    return orc.fmha_i8_blockwise(c["q"], c["k"], c["v"], c["mask"], *_scales(c), block=128 if S % 128 == 0 else 64)
+
+
+# ---- the checker -------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("S,d,pad", [(256, 64, "none"), (192, 128, "scatter"), (384, 64, "scatter")])
+def test_checker_cross_equals_self_on_equal_lengths(orc, S, d, pad):
+    c = fc.make_inputs(2, 2, S, d, pad=pad, seed=31)
+    assert np.array_equal(orc.fmha_i8_blockwise_cross(c["q"], c["k"], c["v"], c["mask"], *_scales(c)), _self(orc, c))
+
+
+@pytest.mark.parametrize("rows", [1, 37, 64, 200])
+def test_checker_fewer_queries_are_a_prefix_of_self_attention(orc, rows):
+    c = fc.make_inputs(2, 3, 256, 64, pad="scatter", seed=32)
+    full = _self(orc, c)
+    got = orc.fmha_i8_blockwise_cross(c["q"][:, :, :rows], c["k"], c["v"], c["mask"], *_scales(c))
+    assert got.shape == (2, 3, rows, 64) and np.array_equal(got, full[:, :, :rows])
+
+
+def test_checker_more_queries_than_keys(orc):
+    # 3 x 128 query rows over 128 keys: each third is a self-attention problem with the same K, V and mask
+    ck = fc.make_inputs(1, 2, 128, 128, pad="scatter", seed=33)
+    qs = [fc.make_inputs(1, 2, 128, 128, seed=40 + i)["q"] for i in range(3)]
+    got = orc.fmha_i8_blockwise_cross(np.concatenate(qs, axis=2), ck["k"], ck["v"], ck["mask"], *_scales(ck))
+    for i, q in enumerate(qs):
+        assert np.array_equal(got[:, :, 128 * i:128 * (i + 1)], _self(orc, dict(ck, q=q)))
+
+
+def test_checker_uniform_attention_closed_form(orc):
+    # Q == 0: every unmasked key weighs the same, O = rne(v_amax/o_amax * mean of the unmasked V rows), for any Sq
+    ck = fc.make_inputs(1, 2, 192, 64, seed=34, valid_lengths=[150])
+    q = np.zeros((1, 2, 77, 64), np.int8)
+    got = orc.fmha_i8_blockwise_cross(q, ck["k"], ck["v"], ck["mask"], 1.0, 1.0, 3.0, 1.5).astype(np.int64)
+    y = 2.0 * ck["v"][:, :, :150].astype(np.float64).mean(axis=2, keepdims=True)
+    want = np.broadcast_to(np.clip(np.rint(y), -127, 127), got.shape)
+    near_tie = np.broadcast_to(np.abs(np.abs(y - np.floor(y)) - 0.5) < 1e-3, got.shape)
+    assert np.array_equal(got[~near_tie], want[~near_tie]) and np.abs(got - want).max() <= 1
+
+
+def test_cross_argument_checks_without_a_gpu(pkg):
+    p = pkg.FMHAParamI8(1.0, 1.0, 1.0, 1.0, 1.0)
+    ok = 0x1000
+
+    def chk(B, Sq, S, H, d, q=ok, k=ok, v=ok, m=ok, o=ok):
+        return pkg.FMHAInferI8CrossCheckArgs(p, pkg.FMHACrossAttnDescriptor(B, Sq, S, H, d), q, k, v, m, o)
+
+    assert chk(1, 1, 64, 1, 64) == pkg.FMHA_I8_OK
+    assert chk(2, 65536, 65536, 3, 128) == pkg.FMHA_I8_OK
+    assert chk(1, 300, 192, 1, 64) == pkg.FMHA_I8_OK
+    assert chk(1, 0, 64, 1, 64) == pkg.FMHA_I8_ERR_SEQ_LEN
+    assert chk(1, 65537, 64, 1, 64) == pkg.FMHA_I8_ERR_SEQ_LEN
+    assert chk(1, 64, 96, 1, 64) == pkg.FMHA_I8_ERR_SEQ_LEN      # keys: multiples of 64 only
+    assert chk(1, 64, 0, 1, 64) == pkg.FMHA_I8_ERR_SEQ_LEN
+    assert chk(1, 64, 64, 1, 96) == pkg.FMHA_I8_ERR_HEAD_DIM
+    assert chk(0, 64, 64, 1, 64) == pkg.FMHA_I8_ERR_BATCH_HEAD
+    assert chk(1, 64, 64, 1, 64, q=ok + 8) == pkg.FMHA_I8_ERR_ALIGNMENT
+    assert chk(1, 64, 64, 1, 64, m=None) == pkg.FMHA_I8_ERR_NULL_POINTER
+
+
+# ---- the HIP kernel ----------------------------------------------------------------------------------------------
+def _gpu(pkg, dev, q, c, canary=False):
+    import torch
+    t = [torch.from_numpy(np.ascontiguousarray(a)).to(dev) for a in (q, c["k"], c["v"], c["mask"])]
+    out = None
+    if canary:
+        # rows past the last query must stay untouched: the output buffer is followed by marked bytes
+        buf = torch.full((q.size + 4096,), 77, dtype=torch.int8, device=dev)
+        out = buf[:q.size].view(q.shape)
+    o = pkg.fmha_infer_i8(*t, *_scales(c), out=out)
+    torch.cuda.synchronize()
+    if canary:
+        assert (buf[q.size:] == 77).all().item()
+    return o.cpu().numpy()
+
+
+def _gate(got, want, what):
+    st = fc.parity_stats(got, want)
+    print(what, st, flush=True)
+    assert st["within1"] >= WITHIN1_MIN and st["max"] <= MAX_ABS_LSB, (what, st)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("Sq,S,pad", [(1, 64, "none"), (31, 128, "scatter"), (33, 192, "scatter"), (100, 512, "none"),
+                                      (256, 128, "scatter"), (257, 320, "tail"), (777, 1024, "scatter"),
+                                      (1024, 64, "none"), (1300, 256, "scatter")])
+def test_cross_attention_against_the_checker(pkg, orc, dev, Sq, S, d, pad):
+    B, H = 2, 3
+    ck = fc.make_inputs(B, H, S, d, pad="scatter" if pad == "scatter" else "none", seed=50,
+                        valid_lengths=[S - 40, S - 64] if pad == "tail" else None)
+    q = fc.make_inputs(B, H, Sq, d, seed=51)["q"]  # quantised normal data, like the keys
+    want = orc.fmha_i8_blockwise_cross(q, ck["k"], ck["v"], ck["mask"], *_scales(ck))
+    _gate(_gpu(pkg, dev, q, ck, canary=True), want, "cross Sq=%d S=%d d=%d %s" % (Sq, S, d, pad))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("S,d", [(512, 128), (320, 64)])
+def test_cross_attention_is_rows_of_self_attention_bit_for_bit(pkg, dev, S, d):
+    """The same kernel computes every query row from the same K, V tiles in the same order whatever the number of
+    rows, so fewer (or regrouped) query rows must reproduce the self-attention bytes exactly."""
+    c = fc.make_inputs(2, 2, S, d, pad="scatter", seed=52)
+    full = _gpu(pkg, dev, c["q"], c)
+    for rows in (1, 32, 45, 256, 300):
+        assert np.array_equal(_gpu(pkg, dev, c["q"][:, :, :rows], c, canary=True), full[:, :, :rows]), rows
+    # more queries than keys: the self-attention queries twice over, the second copy reversed
+    q2 = np.concatenate([c["q"], c["q"][:, :, ::-1]], axis=2)
+    got = _gpu(pkg, dev, q2, c)
+    assert np.array_equal(got[:, :, :S], full) and np.array_equal(got[:, :, S:], full[:, :, ::-1])
+
+
+@pytest.mark.gpu
+def test_cross_attention_decode_shape_at_full_size(pkg, dev):
+    """One query row per head over 65536 keys (the longest key sequence): uniform attention has a closed form."""
+    import torch
+    B, H, S, d = 1, 4, 65536, 64
+    rng = np.random.default_rng(53)
+    v = rng.integers(-127, 128, (B, H, S, d)).astype(np.int8)
+    k = rng.integers(-127, 128, (B, H, S, d)).astype(np.int8)
+    mask = np.zeros((B, S), np.int8)
+    mask[0, 50000:] = 1
+    q = np.zeros((B, H, 1, d), np.int8)
+    c = dict(k=k, v=v, mask=mask, q_amax=1.0, k_amax=1.0, v_amax=40.0, o_amax=1.0)
+    got = _gpu(pkg, dev, q, c, canary=True).astype(np.int64)
+    y = 40.0 * v[:, :, :50000].astype(np.float64).mean(axis=2, keepdims=True)
+    assert np.abs(got - np.clip(np.rint(y), -127, 127)).max() <= 1
+    torch.cuda.synchronize()

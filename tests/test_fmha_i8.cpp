@@ -8,6 +8,7 @@
 //   test_fmha_i8 --sweep                    the reference's own sweep: B=H=1, S in {64,128,...,512,1024,2048,4096}, d in {64,128},
 //                                           uniform(+-0.5) Q/K, |uniform| V, scattered 20 % mask, o_amax measured
 //   test_fmha_i8 --B 2 --H 4 --S 512 --d 64 [--valid L] [--dist normal|student_t|reference]
+//   ... --Sq 100                            that many query rows per head over the S keys (FMHAInferI8Cross)
 //   common: --seed N --iters N --warmup N --cpu-heads N (0 = all) --cpu-threads N --json FILE --no-check
 //   --quant MiB            instead of attention cases: abs-max, quantise and de-quantise (include/fmha_quant.h) over that
 //                          many MiB of fp32 input, checked bit for bit against the CPU checker and timed against HBM
@@ -63,6 +64,7 @@ struct Rng {  // splitmix64 -> uniform -> Box-Muller; identical on every machine
 struct Case {
   std::string name;
   int B = 1, H = 1, S = 128, d = 64;
+  int Sq = 0;                   // query rows per head when they differ from S (0: self-attention, the reference's case)
   std::string dist = "normal";  // normal | student_t | reference
   double sigma = 1.0;
   std::string pad = "none";     // none | bert | tail16th | scatter | valid
@@ -102,9 +104,9 @@ struct Data {
 
 Data generate(const Case& c, uint64_t seed) {
   Data t;
-  const long n = (long)c.B * c.H * c.S * c.d;
-  t.qf.resize(n), t.kf.resize(n), t.vf.resize(n);
-  t.q.resize(n), t.k.resize(n), t.v.resize(n);
+  const long n = (long)c.B * c.H * c.S * c.d, nq = (long)c.B * c.H * (c.Sq > 0 ? c.Sq : c.S) * c.d;
+  t.qf.resize(nq), t.kf.resize(n), t.vf.resize(n);
+  t.q.resize(nq), t.k.resize(n), t.v.resize(n);
   t.mask.assign((long)c.B * c.S, 0);
   Rng rm(seed * 1000003ull + 4), rq(seed * 1000003ull + 1), rk(seed * 1000003ull + 2), rv(seed * 1000003ull + 3);
   for (int b = 0; b < c.B; ++b) {
@@ -115,23 +117,28 @@ Data generate(const Case& c, uint64_t seed) {
     for (int j = 0; j < c.S; ++j)
       t.mask[(long)b * c.S + j] = c.pad == "scatter" ? (rm.uniform() < 0.2 ? 1 : 0) : (j >= L ? 1 : 0);
   }
+  for (long i = 0; i < nq; ++i) {
+    if (c.dist == "reference") t.qf[i] = (float)(rq.uniform() - 0.5);  // test_fmha_i8.cpp:81-89
+    else if (c.dist == "student_t") t.qf[i] = (float)(c.sigma * rq.student_t3());
+    else t.qf[i] = (float)(c.sigma * rq.normal());
+  }
   for (long i = 0; i < n; ++i) {
-    if (c.dist == "reference") {  // test_fmha_i8.cpp:81-89
-      t.qf[i] = (float)(rq.uniform() - 0.5), t.kf[i] = (float)(rk.uniform() - 0.5);
+    if (c.dist == "reference") {
+      t.kf[i] = (float)(rk.uniform() - 0.5);
       t.vf[i] = (float)std::fabs(rv.uniform() - 0.5);
     } else if (c.dist == "student_t") {
-      t.qf[i] = (float)(c.sigma * rq.student_t3()), t.kf[i] = (float)(c.sigma * rk.student_t3());
+      t.kf[i] = (float)(c.sigma * rk.student_t3());
       t.vf[i] = (float)rv.normal();
     } else {
-      t.qf[i] = (float)(c.sigma * rq.normal()), t.kf[i] = (float)(c.sigma * rk.normal());
+      t.kf[i] = (float)(c.sigma * rk.normal());
       t.vf[i] = (float)(c.sigma * rv.normal());
     }
   }
-  t.q_amax = fmha_oracle::abs_max(t.qf.data(), n);  // test_fmha_i8.cpp:95-110
+  t.q_amax = fmha_oracle::abs_max(t.qf.data(), nq);  // test_fmha_i8.cpp:95-110
   t.k_amax = fmha_oracle::abs_max(t.kf.data(), n);
   t.v_amax = fmha_oracle::abs_max(t.vf.data(), n);
+  for (long i = 0; i < nq; ++i) t.q[i] = (int8_t)fmha_oracle::quantize_i8(t.qf[i], t.q_amax);
   for (long i = 0; i < n; ++i) {
-    t.q[i] = (int8_t)fmha_oracle::quantize_i8(t.qf[i], t.q_amax);
     t.k[i] = (int8_t)fmha_oracle::quantize_i8(t.kf[i], t.k_amax);
     t.v[i] = (int8_t)fmha_oracle::quantize_i8(t.vf[i], t.v_amax);
   }
@@ -143,19 +150,23 @@ double seconds_since(std::chrono::steady_clock::time_point t0) {
 }
 
 bool run_case(const Case& c, const Options& opt, FILE* json) {
-  printf("compute type=int32, data type=int8, batch_num=%d, seq_len=%d, head_num=%d, head_dim=%d, dist=%s, pad=%s\n",
+  const bool cross = c.Sq > 0 && c.Sq != c.S;  // queries and keys differ in number: FMHAInferI8Cross
+  const int Sq = cross ? c.Sq : c.S;
+  printf("compute type=int32, data type=int8, batch_num=%d, seq_len=%d, head_num=%d, head_dim=%d, dist=%s, pad=%s",
          c.B, c.S, c.H, c.d, c.dist.c_str(), c.pad.c_str());
+  if (cross) printf(", query rows=%d", Sq);
+  printf("\n");
   fflush(stdout);
   Data t = generate(c, opt.seed);
-  const long n = (long)c.B * c.H * c.S * c.d, heads = (long)c.B * c.H;
+  const long n = (long)c.B * c.H * c.S * c.d, nq = (long)c.B * c.H * Sq * c.d, heads = (long)c.B * c.H;
   const long cpu_heads = (opt.cpu_heads <= 0 || opt.cpu_heads > heads) ? heads : opt.cpu_heads;
   const int threads = opt.cpu_threads > 0 ? opt.cpu_threads : (int)std::thread::hardware_concurrency();
 
   // ---- CPU float path of the reference driver (test_fmha_i8.cpp:141-162), timed, on the sampled heads ------------
-  std::vector<float> o_ref(n, 0.f);
+  std::vector<float> o_ref(nq, 0.f);
   float o_amax = 1.0f;
   double cpu_fp32_s = 0, cpu_i8_s = 0;
-  if (opt.check) {
+  if (opt.check && !cross) {  // (the reference's float path is square: S queries over S keys)
     auto t0 = std::chrono::steady_clock::now();
     fmha_oracle::fmha_fp32_cpu(t.qf.data(), t.kf.data(), t.vf.data(), t.mask.data(), o_ref.data(), c.B, c.H, c.S, c.d,
                                threads, 0, cpu_heads);
@@ -165,13 +176,13 @@ bool run_case(const Case& c, const Options& opt, FILE* json) {
 
   // ---- device buffers, H2D (test_fmha_i8.cpp:165-178) ------------------------------------------------------------
   void *dq, *dk, *dv, *dm, *dout;
-  CHECK_HIP(hipMalloc(&dq, n)), CHECK_HIP(hipMalloc(&dk, n)), CHECK_HIP(hipMalloc(&dv, n));
-  CHECK_HIP(hipMalloc(&dout, n)), CHECK_HIP(hipMalloc(&dm, (size_t)c.B * c.S));
-  CHECK_HIP(hipMemcpy(dq, t.q.data(), n, hipMemcpyHostToDevice));
+  CHECK_HIP(hipMalloc(&dq, nq)), CHECK_HIP(hipMalloc(&dk, n)), CHECK_HIP(hipMalloc(&dv, n));
+  CHECK_HIP(hipMalloc(&dout, nq)), CHECK_HIP(hipMalloc(&dm, (size_t)c.B * c.S));
+  CHECK_HIP(hipMemcpy(dq, t.q.data(), nq, hipMemcpyHostToDevice));
   CHECK_HIP(hipMemcpy(dk, t.k.data(), n, hipMemcpyHostToDevice));
   CHECK_HIP(hipMemcpy(dv, t.v.data(), n, hipMemcpyHostToDevice));
   CHECK_HIP(hipMemcpy(dm, t.mask.data(), (size_t)c.B * c.S, hipMemcpyHostToDevice));
-  CHECK_HIP(hipMemset(dout, 0, n));
+  CHECK_HIP(hipMemset(dout, 0, nq));
   hipStream_t stream;
   CHECK_HIP(hipStreamCreate(&stream));
 
@@ -181,18 +192,25 @@ bool run_case(const Case& c, const Options& opt, FILE* json) {
   desc.batch_num = c.B, desc.seq_len = c.S, desc.head_num = c.H, desc.head_dim = c.d;
   printf("q_amax: %g  k_amax: %g  v_amax: %g  o_amax: %g\n", t.q_amax, t.k_amax, t.v_amax, o_amax);
 
-  const int st = FMHAInferI8Status(stream, param, desc, dq, dk, dv, dm, dout, true);  // warm-up, checked
+  FMHACrossAttnDescriptor xdesc;
+  xdesc.batch_num = c.B, xdesc.seq_len_q = Sq, xdesc.seq_len_kv = c.S, xdesc.head_num = c.H, xdesc.head_dim = c.d;
+  auto call = [&]() {
+    if (cross) (void)FMHAInferI8Cross(stream, param, xdesc, dq, dk, dv, dm, dout);
+    else gpuImpl::FMHAInferI8(stream, param, desc, dq, dk, dv, dm, dout, true);
+  };
+  const int st = cross ? FMHAInferI8Cross(stream, param, xdesc, dq, dk, dv, dm, dout)
+                       : FMHAInferI8Status(stream, param, desc, dq, dk, dv, dm, dout, true);  // warm-up, checked
   if (st != FMHA_I8_OK) {
     fprintf(stderr, "launch failed: %s\n", FMHAInferI8StatusString(st));
     return false;
   }
   // warm-up: the shader clock needs tens of milliseconds of load to settle (a cold call is up to 30 % slower)
-  for (int i = 0; i < opt.warmup; ++i) gpuImpl::FMHAInferI8(stream, param, desc, dq, dk, dv, dm, dout, true);
+  for (int i = 0; i < opt.warmup; ++i) call();
   CHECK_HIP(hipStreamSynchronize(stream));
   hipEvent_t e0, e1;
   CHECK_HIP(hipEventCreate(&e0)), CHECK_HIP(hipEventCreate(&e1));
   CHECK_HIP(hipEventRecord(e0, stream));
-  for (int i = 0; i < opt.iters; ++i) gpuImpl::FMHAInferI8(stream, param, desc, dq, dk, dv, dm, dout, true);
+  for (int i = 0; i < opt.iters; ++i) call();
   CHECK_HIP(hipEventRecord(e1, stream));
   CHECK_HIP(hipEventSynchronize(e1));
   float ms_total = 0;
@@ -201,7 +219,7 @@ bool run_case(const Case& c, const Options& opt, FILE* json) {
   std::vector<float> singles;
   for (int i = 0; i < 20; ++i) {
     CHECK_HIP(hipEventRecord(e0, stream));
-    gpuImpl::FMHAInferI8(stream, param, desc, dq, dk, dv, dm, dout, true);
+    call();
     CHECK_HIP(hipEventRecord(e1, stream));
     CHECK_HIP(hipEventSynchronize(e1));
     float ms1;
@@ -209,15 +227,15 @@ bool run_case(const Case& c, const Options& opt, FILE* json) {
     singles.push_back(ms1 * 1e3f);
   }
   std::sort(singles.begin(), singles.end());
-  const double ops = 4.0 * c.B * c.H * (double)c.S * c.S * c.d;
+  const double ops = 4.0 * c.B * c.H * (double)Sq * c.S * c.d;
   const double tops = ops / us_mean * 1e-6;
   printf("FMHA Inference took %.3f us/call (mean of %d), single-call min %.3f median %.3f us, %.1f TOPS, %.2f %% of "
          "%.1f TOPS int8 peak, %.1f GB/s\n",
          us_mean, opt.iters, singles.front(), singles[singles.size() / 2], tops, 100 * tops / kInt8PeakTops,
-         kInt8PeakTops, (4.0 * n) / us_mean * 1e-3);
+         kInt8PeakTops, (2.0 * n + 2.0 * nq) / us_mean * 1e-3);
 
-  std::vector<int8_t> o(n);
-  CHECK_HIP(hipMemcpy(o.data(), dout, n, hipMemcpyDeviceToHost));
+  std::vector<int8_t> o(nq);
+  CHECK_HIP(hipMemcpy(o.data(), dout, nq, hipMemcpyDeviceToHost));
   CHECK_HIP(hipFree(dq)), CHECK_HIP(hipFree(dk)), CHECK_HIP(hipFree(dv)), CHECK_HIP(hipFree(dm));
   CHECK_HIP(hipFree(dout));
   CHECK_HIP(hipEventDestroy(e0)), CHECK_HIP(hipEventDestroy(e1)), CHECK_HIP(hipStreamDestroy(stream));
@@ -226,12 +244,13 @@ bool run_case(const Case& c, const Options& opt, FILE* json) {
   long hist[4] = {0, 0, 0, 0};
   float dev_pct = 0;
   if (opt.check) {
-    std::vector<int8_t> want(n, 0);
+    std::vector<int8_t> want(nq, 0);
     auto t0 = std::chrono::steady_clock::now();
-    fmha_oracle::fmha_i8_cpu_blockwise(t.q.data(), t.k.data(), t.v.data(), t.mask.data(), want.data(), c.B, c.H, c.S,
-                                       c.d, t.q_amax, t.k_amax, t.v_amax, o_amax, c.S % 128 == 0 ? 128 : 64, threads, 0, cpu_heads);
+    fmha_oracle::fmha_i8_cpu_blockwise_cross(t.q.data(), t.k.data(), t.v.data(), t.mask.data(), want.data(), c.B, c.H,
+                                             Sq, c.S, c.d, t.q_amax, t.k_amax, t.v_amax, o_amax,
+                                             c.S % 128 == 0 ? 128 : 64, threads, 0, cpu_heads);
     cpu_i8_s = seconds_since(t0);
-    const long m = cpu_heads * c.S * c.d;
+    const long m = cpu_heads * Sq * c.d;
     int worst = 0;
     for (long i = 0; i < m; ++i) {
       const int dl = std::abs((int)o[i] - (int)want[i]);
@@ -239,24 +258,25 @@ bool run_case(const Case& c, const Options& opt, FILE* json) {
       worst = std::max(worst, dl);
     }
     const double within1 = (double)(hist[0] + hist[1]) / m;
-    dev_pct = fmha_oracle::mean_rel_deviation_pct(o.data(), o_ref.data(), m, o_amax);  // inc/utils.hpp:59-89
-    pass = within1 >= 0.999 && worst <= 2 && (!c.measured_o_amax || dev_pct < 20.f);
+    if (!cross) dev_pct = fmha_oracle::mean_rel_deviation_pct(o.data(), o_ref.data(), m, o_amax);  // inc/utils.hpp:59-89
+    pass = within1 >= 0.999 && worst <= 2 && (cross || !c.measured_o_amax || dev_pct < 20.f);
     printf("parity vs int8 CPU checker on %ld of %ld heads: delta 0: %ld, 1: %ld, 2: %ld, >2: %ld -> within 1 LSB "
            "%.5f, max %d  [%s]\n", cpu_heads, heads, hist[0], hist[1], hist[2], hist[3], within1, worst,
            pass ? "PASS" : "FAIL");
-    printf("INT8 average absolute deviation vs float path: %f %%%s\n", dev_pct,
-           c.measured_o_amax ? " (reference criterion: < 20)" : " (o_amax fixed at 1: reported only)");
+    if (!cross)
+      printf("INT8 average absolute deviation vs float path: %f %%%s\n", dev_pct,
+             c.measured_o_amax ? " (reference criterion: < 20)" : " (o_amax fixed at 1: reported only)");
     printf("CPU: float path %.3f s, int8 checker %.3f s, %ld heads, %d threads\n", cpu_fp32_s, cpu_i8_s, cpu_heads,
            threads);
   }
   if (json)
     fprintf(json,
-            "{\"case\":\"%s\",\"B\":%d,\"H\":%d,\"S\":%d,\"d\":%d,\"dist\":\"%s\",\"pad\":\"%s\",\"seed\":%llu,"
+            "{\"case\":\"%s\",\"B\":%d,\"H\":%d,\"S\":%d,\"Sq\":%d,\"d\":%d,\"dist\":\"%s\",\"pad\":\"%s\",\"seed\":%llu,"
             "\"mask_polarity\":\"reference (nonzero = masked out)\",\"us_per_call\":%.4f,\"us_single_min\":%.4f,"
             "\"us_single_median\":%.4f,\"tops\":%.3f,\"pct_of_int8_peak\":%.3f,\"iters\":%d,\"checked_heads\":%ld,"
             "\"delta_hist\":[%ld,%ld,%ld,%ld],\"mean_rel_dev_pct\":%.4f,\"cpu_fp32_seconds\":%.4f,"
             "\"cpu_int8_seconds\":%.4f,\"cpu_threads\":%d,\"cpu_heads_extrapolate_factor\":%.3f,\"pass\":%s}\n",
-            c.name.c_str(), c.B, c.H, c.S, c.d, c.dist.c_str(), c.pad.c_str(), (unsigned long long)opt.seed, us_mean,
+            c.name.c_str(), c.B, c.H, c.S, Sq, c.d, c.dist.c_str(), c.pad.c_str(), (unsigned long long)opt.seed, us_mean,
             singles.front(), singles[singles.size() / 2], tops, 100 * tops / kInt8PeakTops, opt.iters,
             opt.check ? cpu_heads : 0, hist[0], hist[1], hist[2], hist[3], dev_pct, cpu_fp32_s, cpu_i8_s, threads,
             (double)heads / cpu_heads, pass ? "true" : "false");
@@ -351,6 +371,7 @@ int main(int argc, char** argv) {
     } else if (a == "--B") custom.B = atoi(val()), have_custom = true;
     else if (a == "--H") custom.H = atoi(val()), have_custom = true;
     else if (a == "--S") custom.S = atoi(val()), have_custom = true;
+    else if (a == "--Sq") custom.Sq = atoi(val()), have_custom = true;
     else if (a == "--d") custom.d = atoi(val()), have_custom = true;
     else if (a == "--valid") custom.valid = atoi(val()), custom.pad = "valid";
     else if (a == "--dist") custom.dist = val();
@@ -370,7 +391,7 @@ int main(int argc, char** argv) {
   }
   if (have_custom) {
     custom.name = "custom";
-    custom.measured_o_amax = custom.dist == "reference";
+    custom.measured_o_amax = custom.dist == "reference" && (custom.Sq == 0 || custom.Sq == custom.S);
     cases.push_back(custom);
   }
   if (cases.empty()) cases.push_back(config_case(1));
