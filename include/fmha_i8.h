@@ -43,7 +43,7 @@ extern "C" {
 #define FMHA_I8_ERR_SEQ_LEN 3        /* key seq_len <= 0, not a multiple of 64, or > 65536; query seq_len <= 0 or > 65536 */
 #define FMHA_I8_ERR_BATCH_HEAD 4     /* batch_num or head_num <= 0, or the grid would exceed HIP limits */
 #define FMHA_I8_ERR_ALIGNMENT 5      /* q, k, v or o not 16-byte aligned */
-#define FMHA_I8_ERR_SCALE 6          /* an amax is not finite, or o_amax <= 0 */
+#define FMHA_I8_ERR_SCALE 6          /* an amax is not finite, o_amax <= 0, or q_amax * k_amax < 0 */
 #define FMHA_I8_ERR_HIP_BASE 1000
 
 /* Replaces gpuImpl::FMHAInferI8 (inc/fmha_i8.h:7-15, src/fmha_i8.cu:157-173).

@@ -32,6 +32,9 @@ int check_args(const FMHAParamI8& p, const FMHACrossAttnDescriptor& a, const voi
   if (bits & 15u) return FMHA_I8_ERR_ALIGNMENT;
   if (!isfinite(p.q_amax) || !isfinite(p.k_amax) || !isfinite(p.v_amax) || !isfinite(p.o_amax) || !(p.o_amax > 0.f))
     return FMHA_I8_ERR_SCALE;
+  // amax values are maxima of absolute values.  The kernel takes row maxima on the integer scores, which is only the
+  // maximum of the scaled scores while the scale is not negative.
+  if (p.q_amax * p.k_amax < 0.f) return FMHA_I8_ERR_SCALE;
   return FMHA_I8_OK;
 }
 
@@ -64,8 +67,10 @@ int launch(hipStream_t stream, const FMHAParamI8& p, const FMHACrossAttnDescript
   const float row_scale = 1.0f / sqrtf((float)a.head_dim);
   const float scale_qk_out = p.q_amax * p.k_amax / (127.f * 127.f);
   args.c2 = row_scale * scale_qk_out * kLog2e;
+  // A masked score is replaced by -inf before it is scaled (see the kernel): the scale must not be exactly 0.  With
+  // 1e-30 every exponent is below 1e-23 in magnitude and the probabilities are the same floats as with 0.
+  if (args.c2 < 1e-30f) args.c2 = 1e-30f;
   args.floor2 = -1e6f * kLog2e;
-  args.masked2 = -1000000.f * args.c2;
   args.out_scale = p.v_amax / (p.o_amax * 128.f);  // inc/fmha_i8.cuh:318
   const dim3 grid((unsigned)args.total_wgs), block(fmha_i8_gfx950::kThreads);
   // The accumulators of Q.K^T can be read as floats without a convert when they start at the bit pattern of kBase;
@@ -133,7 +138,7 @@ const char* FMHAInferI8StatusString(int status) {
     case FMHA_I8_ERR_SEQ_LEN: return "seq_len (of the keys) must be a positive multiple of 64, at most 65536; of the queries 1 to 65536";
     case FMHA_I8_ERR_BATCH_HEAD: return "batch_num and head_num must be positive (and the grid must fit)";
     case FMHA_I8_ERR_ALIGNMENT: return "q, k, v and o must be 16-byte aligned";
-    case FMHA_I8_ERR_SCALE: return "amax values must be finite and o_amax > 0";
+    case FMHA_I8_ERR_SCALE: return "amax values must be finite, o_amax > 0 and q_amax * k_amax >= 0";
     default: break;
   }
   if (status >= FMHA_I8_ERR_HIP_BASE) return hipGetErrorString((hipError_t)(status - FMHA_I8_ERR_HIP_BASE));

@@ -69,7 +69,6 @@ struct KernelArgs {
   int total_wgs;    // batch * head_num * q_blocks
   float c2;         // log2(e) * (1/sqrt(d)) * q_amax*k_amax/127^2 : int32 S -> base-2 exponent
   float floor2;     // log2(e) * -1e6 : the reference's initial block maximum (inc/fmha_i8.cuh:116)
-  float masked2;    // c2 * -1000000 : what a masked key contributes to the block maximum (inc/fmha_i8.cuh:191-193)
   float out_scale;  // v_amax / (o_amax * 128)   (inc/fmha_i8.cuh:318)
 };
 
@@ -84,15 +83,10 @@ __device__ __forceinline__ int v_swizzle(int key) {
   return D == 128 ? ((key & 3) | ((key >> 1) & 4)) : (((key >> 1) & 1) | ((key >> 2) & 2));
 }
 
-// Four floats y_i in [-1, 1] -> four int8 bytes rne(32767 * y_i), packed in order.  v_cvt_pknorm_i16_f32 converts two at a
+// P packing: four floats y_i in [-1, 1] -> four int8 bytes rne(32767 * y_i).  v_cvt_pknorm_i16_f32 converts two at a
 // time (round to nearest; exact .5 ties toward zero, which real softmax values do not hit), v_perm_b32 keeps the low
 // byte of each 16-bit result.
 typedef short v2s __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ int pack4_snorm(float y0, float y1, float y2, float y3) {
-  const v2s lo = __builtin_amdgcn_cvt_pknorm_i16(y0, y1);
-  const v2s hi = __builtin_amdgcn_cvt_pknorm_i16(y2, y3);
-  return __builtin_amdgcn_perm(__builtin_bit_cast(int, hi), __builtin_bit_cast(int, lo), 0x06040200);
-}
 constexpr float kSnorm = 32767.0f;
 
 // Lanes l and l^32 hold the two halves of one query column: v_permlane32_swap hands each lane both halves.
@@ -128,6 +122,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 
   __shared__ __attribute__((aligned(1024))) int8_t lds[kStages][2][kTileBytes];  // [stage][K|V][tile]; tile j -> stage j % kStages
   __shared__ unsigned char lds_class[kMaxKeyBlocks];  // per key block: bit0 = some key masked, bit1 = all keys masked
+  __shared__ unsigned lds_mask[kMaxKeyBlocks * kBlockKSmall / 32];  // bit j%32 of word j/32: key j of this batch entry is masked
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -245,6 +240,12 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     } else if (j < S) {
       nib = (mg[j] != 0 ? 1 : 0) | (mg[j + 1] != 0 ? 2 : 0) | (mg[j + 2] != 0 ? 4 : 0) | (mg[j + 3] != 0 ? 8 : 0);
     }
+    // eight lanes hold the 32 mask bits of one word
+    unsigned word = (unsigned)nib << (4 * (lane & 7));
+    word |= __shfl_xor(word, 1);
+    word |= __shfl_xor(word, 2);
+    word |= __shfl_xor(word, 4);
+    if ((lane & 7) == 0 && j < S) lds_mask[j >> 5] = word;
     const unsigned long long some = __ballot(nib != 0), all = __ballot(nib == 15);
     constexpr int kLanesPerBlock = BK / 4;
     constexpr unsigned long long kBlockBits = (1ull << kLanesPerBlock) - 1;
@@ -338,13 +339,41 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   };
   // (sf(t,r) below: the score as a float; with BIAS that is kBase + S * 2^-26, and the exponent offset removes kBase.)
   // block softmax (inc/fmha_i8.cuh:174-253)
-  auto phase_softmax = [&](int kb, int cls, const v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles], int (&mx)[2]) {
+  auto phase_softmax = [&](int kb, int cls, v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles], int (&mx)[2]) {
     auto sf = [&](int t, int r) -> float { return BIAS ? __int_as_float(acc[t][r]) : (float)acc[t][r]; };
     l_blk = 0.f;
-    if (cls == 0) {
+    if (cls != 0) {
+      // Some keys of this block are masked out (nonzero mask byte, inc/fmha_i8.cuh:189-192,216-221).  Their scores
+      // are replaced by a value that loses every maximum and whose exponential is exactly 0 (-inf read as a float on
+      // the BIAS variant; -2^30 where the scores are converted, which that variant's c2 >= 2.7e-4 turns into an
+      // exponent below -2.9e5), one v_cndmask per score.  The lane masks are wave-uniform - lanes 0..31 hold key
+      // 8a+bb of a tile, lanes 32..63 key 8a+4+bb - so the scalar unit builds them from the block's mask bits.
+      const int gone = BIAS ? (int)0xFF800000 : -(1 << 30);
+#pragma unroll
+      for (int t = 0; t < kKeyTiles; ++t) {
+        const unsigned mw = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_mask[kb * kKeyTiles + t]);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = 8 * (r / 4) + (r % 4);
+          const unsigned lo = (unsigned)(((int)(mw << (31 - key))) >> 31), hi = (unsigned)(((int)(mw << (27 - key))) >> 31);
+          const unsigned long long lanes = ((unsigned long long)hi << 32) | lo;
+          int e = acc[t][r];
+          asm("v_cndmask_b32_e64 %0, %0, %1, %2" : "+v"(e) : "v"(gone), "s"(lanes));
+          acc[t][r] = e;
+        }
+      }
+      // the maximum over the keys that are left (what GEMM 1 collected included the masked ones)
+#pragma unroll
+      for (int t = 0; t + 1 < kKeyTiles; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) tile_max_piece(acc[t], mx, t == 0, j);
+    }
+    {
 #pragma unroll
       for (int j = 0; j < 4; ++j) tile_max_piece(acc[kKeyTiles - 1], mx, false, j);
-      const int ti = half_max(max(mx[0], mx[1]));
+      int ti = half_max(max(mx[0], mx[1]));
+      // a masked key enters the maximum as the integer -1000000 (inc/fmha_i8.cuh:191-193)
+      if (cls != 0) ti = max(ti, (BIAS ? kBaseBits : 0) - 1000000);
       const float top = BIAS ? __int_as_float(ti) : (float)ti;
       // off = top*c2 rounded; p' = exp2(s*c2 - off) = p * 2^(resid) with one row-wide resid below 1 ulp of off, and the
       // block maximum that is consistent with p' is off itself (minus the constant kBase*c2 when BIAS).
@@ -398,42 +427,6 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         if (out) { q_out(s - 1, 5); q_out(s - 1, 6); }
         fence();
       }
-      l_blk = half_sum(l_blk);
-    } else {
-      // some keys of this block are masked out (nonzero mask byte, inc/fmha_i8.cuh:189-192,216-221)
-      const int8_t* mp = mg + kb * BK + 4 * (i32 % (BK / 4));  // lanes past the block re-read it; their bits are not used
-      const int nib = (mp[0] != 0 ? 1 : 0) | (mp[1] != 0 ? 2 : 0) | (mp[2] != 0 ? 4 : 0) | (mp[3] != 0 ? 8 : 0);
-      unsigned mbits[kKeyTiles];  // bit 4a+bb of mbits[t] <-> key 32t + 8a + 4g + bb
-#pragma unroll
-      for (int t = 0; t < kKeyTiles; ++t) {
-        unsigned bits = 0;
-#pragma unroll
-        for (int a = 0; a < 4; ++a) bits |= (unsigned)__shfl(nib, 8 * t + 2 * a + g) << (4 * a);
-        mbits[t] = bits;
-      }
-      const float masked_s = args.masked2 + bias_c2;  // in the units of sf()*c2
-      float top = args.floor2 + bias_c2;
-#pragma unroll
-      for (int t = 0; t < kKeyTiles; ++t)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) top = fmaxf(top, ((mbits[t] >> r) & 1) ? masked_s : sf(t, r) * c2);
-      const float off = half_max(top);
-      m_blk = off - bias_c2;
-      const float offq = off - kLog2Pscale;
-#pragma unroll
-      for (int t = 0; t < kKeyTiles; ++t)
-#pragma unroll
-        for (int a = 0; a < 4; ++a) {
-          float e[4];
-#pragma unroll
-          for (int bb = 0; bb < 4; ++bb) {
-            const int r = 4 * a + bb;
-            const float ex = __builtin_amdgcn_exp2f(__builtin_fmaf(sf(t, r), c2, -offq));
-            e[bb] = ((mbits[t] >> r) & 1) ? 0.f : ex;
-            l_blk += e[bb];
-          }
-          pk[t][a] = pack4_snorm(-e[0], -e[1], -e[2], -e[3]);
-        }
       l_blk = half_sum(l_blk);
     }
   };

@@ -7,7 +7,7 @@
 //   test_fmha_i8 --config 3                 one of the five benchmark configurations
 //   test_fmha_i8 --sweep                    the reference's own sweep: B=H=1, S in {64,128,...,512,1024,2048,4096}, d in {64,128},
 //                                           uniform(+-0.5) Q/K, |uniform| V, scattered 20 % mask, o_amax measured
-//   test_fmha_i8 --B 2 --H 4 --S 512 --d 64 [--valid L] [--dist normal|student_t|reference]
+//   test_fmha_i8 --B 2 --H 4 --S 512 --d 64 [--valid L | --pad none|bert|tail16th|scatter] [--dist normal|student_t|reference]
 //   ... --Sq 100                            that many query rows per head over the S keys (FMHAInferI8Cross)
 //   common: --seed N --iters N --warmup N --cpu-heads N (0 = all) --cpu-threads N --json FILE --no-check
 //   --quant MiB            instead of attention cases: abs-max, quantise and de-quantise (include/fmha_quant.h) over that
@@ -374,6 +374,7 @@ int main(int argc, char** argv) {
     else if (a == "--Sq") custom.Sq = atoi(val()), have_custom = true;
     else if (a == "--d") custom.d = atoi(val()), have_custom = true;
     else if (a == "--valid") custom.valid = atoi(val()), custom.pad = "valid";
+    else if (a == "--pad") custom.pad = val();
     else if (a == "--dist") custom.dist = val();
     else if (a == "--seed") opt.seed = strtoull(val(), nullptr, 10);
     else if (a == "--iters") opt.iters = atoi(val());

@@ -258,6 +258,31 @@ def test_every_kernel_variant(pkg, orc, dev, S, d, qk_scale, vo_ratio):
     check(gpu_run(pkg, dev, c, **kw), cpu_run(orc, c, **kw), "variant S=%d d=%d qk=%g vo=%g" % (S, d, qk_scale, vo_ratio))
 
 
+@pytest.mark.parametrize("S,d", [(256, 128), (192, 64)])
+def test_zero_scale_with_masked_keys(pkg, orc, dev, S, d):
+    """q_amax = 0 (an all-zero Q tensor quantised by abs-max): every score scales to 0, the softmax is uniform over the
+    unmasked keys, and a masked key must still weigh exactly nothing."""
+    c = fc.make_inputs(1, 2, S, d, pad="scatter", seed=46)
+    got = gpu_run(pkg, dev, c, q_amax=0.0, v_amax=2.0, o_amax=1.0).astype(np.int64)
+    keep = c["mask"][0] == 0
+    y = 2.0 * c["v"][:, :, keep, :].astype(np.float64).mean(axis=2, keepdims=True)
+    assert np.abs(got - np.clip(np.rint(y), -127, 127)).max() <= 1
+    check(got, cpu_run(orc, c, q_amax=0.0, v_amax=2.0, o_amax=1.0), "zero scale S=%d d=%d" % (S, d))
+
+
+def test_negative_score_scale_is_refused(pkg, dev):
+    import torch
+    c = fc.make_inputs(1, 1, 128, 64, seed=47)
+    q, k, v, m = to_dev(dev, c["q"], c["k"], c["v"], c["mask"])
+    o = torch.full_like(q, 55)
+    P = pkg.FMHAParamI8(-1.0, 1.0, 1.0, 1.0, 1.0)
+    assert pkg.FMHAInferI8Status(None, P, pkg.AttnDataDescriptor(1, 128, 1, 64), q, k, v, m, o) == pkg.FMHA_I8_ERR_SCALE
+    P = pkg.FMHAParamI8(-1.0, -1.0, 1.0, 1.0, 1.0)  # the product is what scales the scores
+    assert pkg.FMHAInferI8CheckArgs(P, pkg.AttnDataDescriptor(1, 128, 1, 64), q, k, v, m, o) == pkg.FMHA_I8_OK
+    torch.cuda.synchronize()
+    assert (o == 55).all().item()
+
+
 def test_masked_sentinel_corner(pkg, orc, dev):
     # every unmasked score of a partially masked block lies below the -1,000,000 substituted for masked keys
     S, d = 128, 128
