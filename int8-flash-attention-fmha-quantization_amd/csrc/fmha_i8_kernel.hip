@@ -45,9 +45,9 @@ constexpr int kStages = 4;     // K/V tiles resident in LDS per kind: a tile is 
 constexpr int kXcds = 8;
 constexpr int kMaxKeyBlocks = 1024;      // seq_len <= 65536, also in blocks of 64 keys
 constexpr float kMagic = 12582912.0f;    // 1.5 * 2^23: kMagic + y holds rne(y) in its low mantissa bits (output rounding)
-// Both GEMMs start their int32 accumulators at the bit pattern of the float 1/(2 pi), which the MFMA takes as an INLINE
-// CONSTANT C operand (no registers, no moves).  That float sits 2292099 ulps above 2^-3 and 6096509 below 2^-2, more than
-// any int8 dot product of 128 terms can reach (|x| <= 2^21), so kBaseBits + x read as a float is exactly
+// Both GEMMs start their int32 accumulators at the bit pattern of the float 1/(2 pi), held in sixteen registers that
+// the first MFMA of every chain names as its C operand.  That float sits 2292099 ulps above 2^-3 and 6096509 below 2^-2,
+// more than any int8 dot product of 128 terms can reach (|x| <= 2^21), so kBaseBits + x read as a float is exactly
 // kBase + x * 2^-26: the integer result is available to float arithmetic without a convert.
 constexpr int kBaseBits = 0x3E22F983;
 constexpr float kBase = __builtin_bit_cast(float, kBaseBits);
@@ -276,8 +276,9 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   const float bias_c2 = BIAS ? kBase * c2 : 0.f;
   float magic = kMagic;
   asm volatile("" : "+v"(magic));  // a register operand: as a literal it would double the size of every instruction using it
-  const v16i base_c = {kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits,
-                       kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits};
+  v16i base_c = {kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits,
+                 kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits};
+  asm volatile("" : "+v"(base_c));  // held in registers: as a known constant it is rebuilt by eight moves per key block
 
   // K0 and Q have landed once at most V0 is still in flight.  The registers are redefined after the wait so that no
   // use of them can be scheduled above it.
