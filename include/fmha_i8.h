@@ -15,11 +15,13 @@
  *   asynchrony     one kernel is enqueued on `stream`; the call returns immediately and never synchronises.
  *   threading      no mutable global state: callable concurrently from any host thread.
  *
- * Supported shapes: head_dim in {64, 128}; seq_len a positive multiple of 64, at most 65536; batch_num, head_num >= 1.
+ * Supported shapes: head_dim in {64, 128}; seq_len from 1 to 65536; batch_num, head_num >= 1.
  * (The reference's ladder, src/fmha_i8.cu:39-154, covers head_dim in {64,128} and eleven fixed seq_len values: 64, 128,
- * 192, 256, 320, 384, 448, 512, 1024, 2048, 4096.  All of them are covered here, and so is every other multiple of 64.
+ * 192, 256, 320, 384, 448, 512, 1024, 2048, 4096.  All of them are covered here, and so is every other length.
  * As in the reference, the softmax works on blocks of 128 keys when seq_len is a multiple of 128 and on blocks of 64 keys
- * otherwise - the block size is part of the numerics, because P is quantised against the BLOCK-LOCAL row maximum.)
+ * when it is another multiple of 64 - the block size is part of the numerics, because P is quantised against the
+ * BLOCK-LOCAL row maximum.  A length that is not a multiple of 64 gives exactly what the caller would get by padding
+ * K, V and the mask to the next multiple of 64 with masked keys; the library does it without the copies.)
  *
  * Numerics follow the reference kernel (inc/fmha_i8.cuh:71-72,181-253,298-332): int32 Q.K^T, 1/sqrt(d) and
  * q_amax*k_amax/127^2 dequantisation, softmax over blocks of 128 (or 64) keys with the BLOCK-LOCAL row maximum,
@@ -40,7 +42,7 @@ extern "C" {
 #define FMHA_I8_OK 0
 #define FMHA_I8_ERR_NULL_POINTER 1   /* q, k, v, padding_mask or o is NULL */
 #define FMHA_I8_ERR_HEAD_DIM 2       /* head_dim not in {64, 128} */
-#define FMHA_I8_ERR_SEQ_LEN 3        /* key seq_len <= 0, not a multiple of 64, or > 65536; query seq_len <= 0 or > 65536 */
+#define FMHA_I8_ERR_SEQ_LEN 3        /* a seq_len (queries or keys) <= 0 or > 65536 */
 #define FMHA_I8_ERR_BATCH_HEAD 4     /* batch_num or head_num <= 0, or the grid would exceed HIP limits */
 #define FMHA_I8_ERR_ALIGNMENT 5      /* q, k, v or o not 16-byte aligned */
 #define FMHA_I8_ERR_SCALE 6          /* an amax is not finite, o_amax <= 0, or q_amax * k_amax < 0 */
@@ -70,7 +72,7 @@ int FMHAInferI8CheckArgs(FMHAParamI8 fmha_param, AttnDataDescriptor attn_desc, c
 typedef struct FMHACrossAttnDescriptor {
   int batch_num;
   int seq_len_q;   /* rows of q and o per head: any count from 1 to 65536 */
-  int seq_len_kv;  /* rows of k and v per head, and mask bytes per batch entry: a positive multiple of 64, <= 65536 */
+  int seq_len_kv;  /* rows of k and v per head, and mask bytes per batch entry: any count from 1 to 65536 */
   int head_num;
   int head_dim;
 } FMHACrossAttnDescriptor;
@@ -78,7 +80,7 @@ typedef struct FMHACrossAttnDescriptor {
 /* Attention of seq_len_q queries over seq_len_kv keys.  q, o: int8 [batch_num, head_num, seq_len_q, head_dim];
  * k, v: int8 [batch_num, head_num, seq_len_kv, head_dim]; padding_mask: int8 [batch_num, seq_len_kv].  Everything
  * else (scales, numerics, ownership, asynchrony, status codes) as for FMHAInferI8Status; the softmax block is 128 keys
- * when seq_len_kv is a multiple of 128, else 64.  Query rows are independent of each other, so with
+ * when seq_len_kv, rounded up to a multiple of 64, is a multiple of 128, else 64.  Query rows are independent of each other, so with
  * seq_len_q == seq_len_kv this IS FMHAInferI8Status (same kernel, same launch), and a call on the first n query rows
  * of a self-attention problem gives the first n rows of its output. */
 int FMHAInferI8Cross(hipStream_t stream, FMHAParamI8 fmha_param, FMHACrossAttnDescriptor desc, const void* q,

@@ -22,9 +22,7 @@ int check_args(const FMHAParamI8& p, const FMHACrossAttnDescriptor& a, const voi
                const void* mask, const void* o) {
   if (!q || !k || !v || !mask || !o) return FMHA_I8_ERR_NULL_POINTER;
   if (a.head_dim != 64 && a.head_dim != 128) return FMHA_I8_ERR_HEAD_DIM;
-  if (a.seq_len_kv <= 0 || a.seq_len_kv % fmha_i8_gfx950::kBlockKSmall != 0 || a.seq_len_kv > 65536)
-    return FMHA_I8_ERR_SEQ_LEN;
-  if (a.seq_len_q <= 0 || a.seq_len_q > 65536) return FMHA_I8_ERR_SEQ_LEN;
+  if (a.seq_len_kv <= 0 || a.seq_len_kv > 65536 || a.seq_len_q <= 0 || a.seq_len_q > 65536) return FMHA_I8_ERR_SEQ_LEN;
   if (a.batch_num <= 0 || a.head_num <= 0) return FMHA_I8_ERR_BATCH_HEAD;
   const long long wgs = (long long)a.batch_num * a.head_num * ((a.seq_len_q + fmha_i8_gfx950::kBlockQ - 1) / fmha_i8_gfx950::kBlockQ);
   if (wgs > 0x7fffffffLL) return FMHA_I8_ERR_BATCH_HEAD;
@@ -38,13 +36,18 @@ int check_args(const FMHAParamI8& p, const FMHACrossAttnDescriptor& a, const voi
   return FMHA_I8_OK;
 }
 
-template <int D, int BK>
-void launch_variant(bool bias, bool fast, dim3 grid, dim3 block, hipStream_t stream, const fmha_i8_gfx950::KernelArgs& args) {
+template <int D, int BK, bool RAGGED>
+void launch_variant3(bool bias, bool fast, dim3 grid, dim3 block, hipStream_t stream, const fmha_i8_gfx950::KernelArgs& args) {
   using namespace fmha_i8_gfx950;
-#define FMHA_LAUNCH(BB, FF) hipLaunchKernelGGL((fmha_i8_fwd_kernel<D, BK, BB, FF>), grid, block, 0, stream, args)
+#define FMHA_LAUNCH(BB, FF) hipLaunchKernelGGL((fmha_i8_fwd_kernel<D, BK, BB, FF, RAGGED>), grid, block, 0, stream, args)
   if (bias) { if (fast) FMHA_LAUNCH(true, true); else FMHA_LAUNCH(true, false); }
   else { if (fast) FMHA_LAUNCH(false, true); else FMHA_LAUNCH(false, false); }
 #undef FMHA_LAUNCH
+}
+template <int D, int BK>
+void launch_variant(bool bias, bool fast, dim3 grid, dim3 block, hipStream_t stream, const fmha_i8_gfx950::KernelArgs& args) {
+  if (args.seq_kv % BK != 0) launch_variant3<D, BK, true>(bias, fast, grid, block, stream, args);
+  else launch_variant3<D, BK, false>(bias, fast, grid, block, stream, args);
 }
 
 int launch(hipStream_t stream, const FMHAParamI8& p, const FMHACrossAttnDescriptor& a, const void* q, const void* k,
@@ -83,8 +86,10 @@ int launch(hipStream_t stream, const FMHAParamI8& p, const FMHACrossAttnDescript
   // LSBs that is at most about 0.0034 * (v_amax/o_amax) * sqrt(key blocks).  Take it while that stays below 0.1 LSB.
   // Blocks of 128 keys, as the reference uses for its multiples of 128; its other lengths (64, 192, 320, 448:
   // src/fmha_i8.cu:41-60) run in blocks of 64 keys, and so does every other odd multiple of 64 here.
-  const int block_keys = a.seq_len_kv % fmha_i8_gfx950::kBlockK == 0 ? fmha_i8_gfx950::kBlockK : fmha_i8_gfx950::kBlockKSmall;
-  const float lsb_bound = 0.0034f * fabsf(p.v_amax / p.o_amax) * sqrtf((float)(a.seq_len_kv / block_keys));
+  // A key count that is not a multiple of 64 is treated as the next multiple of 64 whose last keys are masked out.
+  const int kv_padded = (a.seq_len_kv + fmha_i8_gfx950::kBlockKSmall - 1) / fmha_i8_gfx950::kBlockKSmall * fmha_i8_gfx950::kBlockKSmall;
+  const int block_keys = kv_padded % fmha_i8_gfx950::kBlockK == 0 ? fmha_i8_gfx950::kBlockK : fmha_i8_gfx950::kBlockKSmall;
+  const float lsb_bound = 0.0034f * fabsf(p.v_amax / p.o_amax) * sqrtf((float)(kv_padded / block_keys));
   const bool fast = lsb_bound < 0.1f;
   if (a.head_dim == 128) {
     if (block_keys == fmha_i8_gfx950::kBlockK) launch_variant<128, fmha_i8_gfx950::kBlockK>(bias, fast, grid, block, stream, args);
@@ -135,7 +140,7 @@ const char* FMHAInferI8StatusString(int status) {
     case FMHA_I8_OK: return "ok";
     case FMHA_I8_ERR_NULL_POINTER: return "null pointer argument";
     case FMHA_I8_ERR_HEAD_DIM: return "head_dim must be 64 or 128";
-    case FMHA_I8_ERR_SEQ_LEN: return "seq_len (of the keys) must be a positive multiple of 64, at most 65536; of the queries 1 to 65536";
+    case FMHA_I8_ERR_SEQ_LEN: return "seq_len must be between 1 and 65536 (queries and keys alike)";
     case FMHA_I8_ERR_BATCH_HEAD: return "batch_num and head_num must be positive (and the grid must fit)";
     case FMHA_I8_ERR_ALIGNMENT: return "q, k, v and o must be 16-byte aligned";
     case FMHA_I8_ERR_SCALE: return "amax values must be finite, o_amax > 0 and q_amax * k_amax >= 0";

@@ -63,7 +63,8 @@ struct KernelArgs {
   const int8_t* mask;
   int8_t* o;
   int seq_q;        // query (and output) rows per head: any positive count
-  int seq_kv;       // key/value rows per head and mask bytes per batch entry: a multiple of BK
+  int seq_kv;       // key/value rows per head and mask bytes per batch entry: any positive count; keys from there to
+                    // the next multiple of BK do not exist and count as masked
   int head_num;
   int q_blocks;     // ceil(seq_q / kBlockQ)
   int total_wgs;    // batch * head_num * q_blocks
@@ -108,7 +109,9 @@ __device__ __forceinline__ float half_sum(float x) {
 // FASTACC: the running O absorbs the kBase offset of the GEMM 2 accumulators (one fma per element and key block
 // instead of subtract + fma) and the offset is taken out once, in the epilogue.  O then lives near kBase * sum(take)
 // and each merge rounds at that magnitude; the host enables it only where that rounding is far below one output LSB.
-template <int D, int BK, bool BIAS, bool FASTACC>
+// RAGGED: seq_kv is not a multiple of BK.  Everything that serves the partly filled last block is compiled in only
+// then: in the key loop it costs some fifty scalar instructions per block, which the other lengths do not pay.
+template <int D, int BK, bool BIAS, bool FASTACC, bool RAGGED>
 __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelArgs args) {
   constexpr int kChunks = D / 16;                     // 16-byte chunks per row
   constexpr int kTileBytes = BK * D;                  // one K or V tile
@@ -147,7 +150,16 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   const int8_t* __restrict__ kg = args.k + head_off;
   const int8_t* __restrict__ vg = args.v + head_off;
   const int8_t* __restrict__ mg = args.mask + (long)b * S;
-  const int n_blocks = S / BK;
+  const int n_blocks = (S + BK - 1) / BK;
+  const int S_pad = n_blocks * BK;
+  // A last key block that is only partly there: its tile loads must not run past the end of K and V.  When it is
+  // not the only block its tiles are fetched from BK rows earlier than their place, so that they END with the last key
+  // (a change of the wave-uniform base address and nothing else): LDS row r then holds key S - BK + r, the first
+  // BK - tail_rows rows repeat keys of the block before and are masked like the padding they stand for.  A sequence
+  // shorter than one block is fetched in the prologue with the rows past its end redirected to its last key.
+  const int tail_rows = S - (n_blocks - 1) * BK;
+  const int tail_kb = (RAGGED && n_blocks > 1) ? n_blocks - 1 : -1;  // the block with the shifted window
+  const bool short_seq = RAGGED && S < BK;
 
   // The prologue puts every cold miss in flight before it waits for any of them: the mask bytes, the first two K/V
   // tiles (tile 1 on speculation: it exists whenever seq_kv >= 256, whether or not its keys are masked) and the Q rows.
@@ -155,8 +167,9 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // direct-to-LDS loads: lane l of a 1 KiB region lands at byte 16*l of the region, so the lane FETCHES the chunk that
   // the swizzle assigns to that slot.
   int ld_goff_k, ld_goff_v;
+  const int ld_row_in = lane / kChunks;
   {
-    const int row_in = lane / kChunks, p = lane % kChunks;
+    const int row_in = ld_row_in, p = lane % kChunks;
     const int vrow = (D == 128) ? (row_in | ((wave & 1) << 3)) : row_in;  // row bits the V swizzle looks at
     ld_goff_k = row_in * D + ((p ^ k_swizzle<D>(row_in)) << 4);
     ld_goff_v = row_in * D + ((p ^ v_swizzle<D>(vrow)) << 4);
@@ -182,6 +195,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) int8_t*)&lds[0][0][0];
   auto issue_tile = [&](const int8_t* gbase, int kb, int which, int goff) {  // which: 0 = K, 1 = V
     const int8_t* gp = gbase + (long)kb * kTileBytes;  // wave-uniform base (SGPR pair)
+    if (RAGGED && kb == tail_kb) gp = gbase + (long)(S - BK) * D;
 #pragma unroll
     for (int it = 0; it < kRegionsPerWave; ++it) {
       const int region = (it * kWaves + wave) % kRegions;
@@ -192,6 +206,19 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   };
   auto issue_k = [&](int kb) { issue_tile(kg, kb, 0, ld_goff_k); };
   auto issue_v = [&](int kb) { issue_tile(vg, kb, 1, ld_goff_v); };
+  // tile 0 of a sequence shorter than one block (prologue only): rows past the last key fetch the last key instead
+  // (same chunk: the swizzle belongs to the LDS row); what lands there is never attended to, those keys are masked
+  auto issue_short = [&](const int8_t* gbase, int which, int goff) {
+#pragma unroll
+    for (int it = 0; it < kRegionsPerWave; ++it) {
+      const int region = (it * kWaves + wave) % kRegions;
+      const unsigned dst = lds_base + (unsigned)(which * kTileBytes + region * 1024);
+      const int row = region * kRowsPerRegion + ld_row_in;
+      const int src = goff + region * 1024 - (row >= S ? (row - (S - 1)) * D : 0);
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                   :: "s"(dst), "v"(src), "s"(gbase) : "memory");
+    }
+  };
   // Memory reads return in issue order: waiting until at most `tiles` tiles of this wavefront's loads are outstanding
   // retires every tile older than the newest `tiles` ones.
   auto wait_all_but = [&](int tiles) {
@@ -211,12 +238,13 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // everything queued here delays the first GEMM.)
   const int row0 = qb * kBlockQ + wave * 32;  // first query row of this wavefront
   const bool active = row0 < Sq;              // the last workgroup of a head may be partly empty
-  int mask_word;
-  {
-    const int j = 4 * tid < S ? 4 * tid : S - 4;
+  int mask_word = 0;
+  if (!RAGGED || S >= 4) {  // (a shorter mask row has no dword that lies inside it)
+    const int j = 4 * tid + 4 <= S ? 4 * tid : S - 4;
     asm volatile("global_load_dword %0, %1, %2" : "=v"(mask_word) : "v"(j), "s"(mg) : "memory");
   }
-  issue_k(0);
+  if (short_seq) issue_short(kg, 0, ld_goff_k);
+  else issue_k(0);
   v4i qreg[kDSteps];  // Q: B operand of GEMM 1, loaded once
   {
     // rows past the end of the sequence load the last row (unused) so that every wavefront has the same loads in flight
@@ -227,34 +255,57 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     for (int kk = 0; kk < kDSteps; ++kk)
       asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(qreg[kk]) : "v"(qoff + 32 * kk), "s"(qp) : "memory");
   }
-  issue_v(0);
+  if (short_seq) issue_short(vg, 1, ld_goff_v);
+  else issue_v(0);
 
   // ---- classify the key blocks of this batch entry: 4 mask bytes per lane, BK/4 lanes per block ---------------------
   asm volatile("s_waitcnt vmcnt(%1)" : "+v"(mask_word) : "n"(2 * kRegionsPerWave + kDSteps) : "memory");
-  for (int base = 0; base < S; base += 4 * kThreads) {
+  for (int base = 0; base < S_pad; base += 4 * kThreads) {
     const int j = base + 4 * tid;
-    int nib = 15;
-    if (base == 0) {
-      const unsigned w = (unsigned)mask_word;
-      if (j < S) nib = ((w & 0xffu) ? 1 : 0) | ((w & 0xff00u) ? 2 : 0) | ((w & 0xff0000u) ? 4 : 0) | ((w & 0xff000000u) ? 8 : 0);
-    } else if (j < S) {
-      nib = (mg[j] != 0 ? 1 : 0) | (mg[j + 1] != 0 ? 2 : 0) | (mg[j + 2] != 0 ? 4 : 0) | (mg[j + 3] != 0 ? 8 : 0);
+    int nib = 15;  // keys past the end of the sequence count as masked
+    if (RAGGED ? j + 4 <= S : j < S) {
+      if (base == 0) {
+        const unsigned w = (unsigned)mask_word;
+        nib = ((w & 0xffu) ? 1 : 0) | ((w & 0xff00u) ? 2 : 0) | ((w & 0xff0000u) ? 4 : 0) | ((w & 0xff000000u) ? 8 : 0);
+      } else {
+        nib = (mg[j] != 0 ? 1 : 0) | (mg[j + 1] != 0 ? 2 : 0) | (mg[j + 2] != 0 ? 4 : 0) | (mg[j + 3] != 0 ? 8 : 0);
+      }
+    } else if (RAGGED && j < S) {  // the one lane that straddles the end
+      for (int b = 0; b < S - j; ++b) nib = (mg[j + b] != 0) ? nib : (nib & ~(1 << b));
     }
     // eight lanes hold the 32 mask bits of one word
     unsigned word = (unsigned)nib << (4 * (lane & 7));
     word |= __shfl_xor(word, 1);
     word |= __shfl_xor(word, 2);
     word |= __shfl_xor(word, 4);
-    if ((lane & 7) == 0 && j < S) lds_mask[j >> 5] = word;
+    if ((lane & 7) == 0 && j < S_pad) lds_mask[j >> 5] = word;
     const unsigned long long some = __ballot(nib != 0), all = __ballot(nib == 15);
     constexpr int kLanesPerBlock = BK / 4;
     constexpr unsigned long long kBlockBits = (1ull << kLanesPerBlock) - 1;
-    if (lane % kLanesPerBlock == 0 && j < S) {
+    if (lane % kLanesPerBlock == 0 && j < S_pad) {
       const unsigned long long blk_some = (some >> lane) & kBlockBits, blk_all = (all >> lane) & kBlockBits;
       lds_class[j / BK] = (unsigned char)((blk_some != 0 ? 1 : 0) | (blk_all == kBlockBits ? 2 : 0));
     }
   }
   __syncthreads();
+  // mask bits of the shifted last block: bit r of word t <-> key S - BK + 32 t + r; the repeated keys count as masked
+  unsigned tail_word[kKeyTiles];
+#pragma unroll
+  for (int t = 0; t < kKeyTiles; ++t) tail_word[t] = 0;
+  if (RAGGED && tail_kb >= 0) {
+    const int repeated = BK - tail_rows;
+#pragma unroll
+    for (int t = 0; t < kKeyTiles; ++t) {
+      const int start = S - BK + 32 * t, w = start >> 5, sh = start & 31;
+      const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_mask[w]);
+      const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_mask[w + (sh ? 1 : 0)]);
+      unsigned word = sh ? (lo >> sh) | (hi << (32 - sh)) : lo;
+      const int forced = repeated - 32 * t;  // leading bits of this word that belong to repeated keys
+      if (forced >= 32) word = 0xffffffffu;
+      else if (forced > 0) word |= (1u << forced) - 1u;
+      tail_word[t] = word;
+    }
+  }
   // last key block that holds any unmasked key (trailing padding is never computed on)
   int last_block = -1;
   for (int base = 0; base < n_blocks; base += 64) {
@@ -352,7 +403,9 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       const int gone = BIAS ? (int)0xFF800000 : -(1 << 30);
 #pragma unroll
       for (int t = 0; t < kKeyTiles; ++t) {
-        const unsigned mw = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_mask[kb * kKeyTiles + t]);
+        const unsigned mw = (RAGGED && kb == tail_kb)
+                                ? tail_word[t]
+                                : (unsigned)__builtin_amdgcn_readfirstlane((int)lds_mask[kb * kKeyTiles + t]);
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = 8 * (r / 4) + (r % 4);

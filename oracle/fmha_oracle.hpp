@@ -152,7 +152,8 @@ inline void parallel_for(long n, int threads, F&& body) {
 //   q, o : int8 [Sq][d] of this head.  The reference has Sq == S only (one SEQ_LEN sizes everything, fmha_i8.cuh:45);
 //          each query row is processed on its own below, as it is in the reference (a warp's 16 rows share nothing
 //          but the K/V tiles), so any Sq is the same arithmetic applied to another number of rows.
-//   block      : keys per softmax block (BASE_SEQ_LEN: 128, or 64 for the reference's 64-multiples)
+//   block      : keys per softmax block (BASE_SEQ_LEN: 128, or 64 for the reference's 64-multiples); for a key count
+//                that is no multiple of 64 the caller passes the block of the next multiple of 64
 // Differences from the reference kernel, both deliberate and both outside what its own test exercises:
 //   * a key block with every key masked is skipped (reference: harmless when it is not the first block, NaN when it
 //     is, fmha_i8.cuh:91-92,116-117,301-310);
@@ -187,7 +188,9 @@ inline void fmha_i8_head_blockwise(const int8_t* q, const int8_t* k, const int8_
       }
       // Block-local row max (fmha_i8.cuh:116,181-206): masked keys enter as the integer -1000000; the max starts
       // at -1e6f; value = (row_scale * float(int)) * scale_qk_out, which is monotone in the integer.
-      int top_int = std::numeric_limits<int>::min();
+      // A last block that is only partly there (a key count that is no multiple of the block; the reference has no
+      // such length, src/fmha_i8.cu:39-154) is a full block whose missing keys are masked: they enter the maximum too.
+      int top_int = nb < block ? kMaskedInt : std::numeric_limits<int>::min();
       for (int j = 0; j < nb; ++j) top_int = std::max(top_int, mask[k0 + j] ? kMaskedInt : s_int[j]);
       const float m_blk = std::max(-1e6f, row_scale * static_cast<float>(top_int) * scale_qk_out);
       // exp and un-quantised row sum (fmha_i8.cuh:208-235); a*b - c contracts to one fma under nvcc's default.

@@ -148,16 +148,18 @@ def fmha_i8_blockwise(q, k, v, mask, q_amax, k_amax, v_amax, o_amax, block=128, 
 
 def fmha_i8_blockwise_cross(q, k, v, mask, q_amax, k_amax, v_amax, o_amax, block=None, threads=None):
     """q: int8 [B,H,Sq,d]; k, v: int8 [B,H,S,d]; mask: int8 [B,S], nonzero = masked out.  Returns int8 O [B,H,Sq,d].
-    block defaults to what the reference's ladder would give S: 128 keys for multiples of 128, else 64."""
+    block defaults to what the reference's ladder would give S: 128 keys for multiples of 128, else 64.  A key count
+    that is no multiple of 64 means the next multiple of 64 with the missing keys masked out."""
     B, H, Sq, d = q.shape
     S = k.shape[2]
+    assert k.shape == (B, H, S, d) and v.shape == k.shape and mask.shape == (B, S)
     q, k, v = (np.ascontiguousarray(t, dtype=np.int8) for t in (q, k, v))
     mask = np.ascontiguousarray(mask, dtype=np.int8)
-    assert k.shape == (B, H, S, d) and v.shape == k.shape and mask.shape == (B, S)
     o = np.zeros_like(q)
     lib().oracle_fmha_i8_blockwise_cross(q.reshape(-1), k.reshape(-1), v.reshape(-1), mask.reshape(-1), o.reshape(-1),
                                          B, H, Sq, S, d, q_amax, k_amax, v_amax, o_amax,
-                                         block or (128 if S % 128 == 0 else 64), threads or hardware_threads(),
+                                         block or (128 if (S + 63) // 64 * 64 % 128 == 0 else 64),
+                                         threads or hardware_threads(),
                                          0, B * H)
     return o
 

@@ -70,7 +70,8 @@ def test_cross_argument_checks_without_a_gpu(pkg):
     assert chk(1, 300, 192, 1, 64) == pkg.FMHA_I8_OK
     assert chk(1, 0, 64, 1, 64) == pkg.FMHA_I8_ERR_SEQ_LEN
     assert chk(1, 65537, 64, 1, 64) == pkg.FMHA_I8_ERR_SEQ_LEN
-    assert chk(1, 64, 96, 1, 64) == pkg.FMHA_I8_ERR_SEQ_LEN      # keys: multiples of 64 only
+    assert chk(1, 64, 96, 1, 64) == pkg.FMHA_I8_OK                # any key count
+    assert chk(1, 64, 65537, 1, 64) == pkg.FMHA_I8_ERR_SEQ_LEN
     assert chk(1, 64, 0, 1, 64) == pkg.FMHA_I8_ERR_SEQ_LEN
     assert chk(1, 64, 64, 1, 96) == pkg.FMHA_I8_ERR_HEAD_DIM
     assert chk(0, 64, 64, 1, 64) == pkg.FMHA_I8_ERR_BATCH_HEAD
@@ -145,3 +146,66 @@ def test_cross_attention_decode_shape_at_full_size(pkg, dev):
     y = 40.0 * v[:, :, :50000].astype(np.float64).mean(axis=2, keepdims=True)
     assert np.abs(got - np.clip(np.rint(y), -127, 127)).max() <= 1
     torch.cuda.synchronize()
+
+
+# ---- key counts that are not multiples of 64 -----------------------------------------------------------------------
+def test_checker_ragged_key_count_means_padding_with_masked_keys(orc):
+    c = fc.make_inputs(1, 2, 192, 64, pad="scatter", seed=60)
+    q = c["q"][:, :, :50]
+    for S in (129, 150, 191):
+        got = orc.fmha_i8_blockwise_cross(q, c["k"][:, :, :S], c["v"][:, :, :S], c["mask"][:, :S], *_scales(c))
+        m = c["mask"].copy()
+        m[:, S:] = 1  # same keys, the rest masked: what lies in K and V behind a masked key cannot matter
+        assert np.array_equal(got, orc.fmha_i8_blockwise_cross(q, c["k"], c["v"], m, *_scales(c))), S
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("S", [1, 3, 4, 5, 63, 65, 100, 127, 129, 191, 193, 255, 257, 1000, 1023, 1025, 2049])
+def test_any_key_count(pkg, orc, dev, S, d):
+    """Self-attention and cross-attention with a key count that is no multiple of 64: the HIP kernel against the
+    checker (gate), and against itself on inputs that the caller padded to the next multiple of 64 with masked keys
+    and other bytes in the padding (so a read of padding that reaches the output shows)."""
+    B, H = 2, 2
+    Sp = (S + 63) // 64 * 64
+    c = fc.make_inputs(B, H, Sp, d, pad="scatter" if S > 8 else "none", seed=61)
+    if S > 8:
+        c["mask"][:, 0] = 0  # at least one key that every batch entry attends to
+    cut = dict(c, k=c["k"][:, :, :S], v=c["v"][:, :, :S], mask=c["mask"][:, :S])
+    cut = {n: (np.ascontiguousarray(a) if isinstance(a, np.ndarray) else a) for n, a in cut.items()}
+    padded = dict(c, mask=c["mask"].copy())
+    padded["mask"][:, S:] = 1
+    for Sq in sorted({S, 77}):
+        q = fc.make_inputs(B, H, Sq, d, seed=62)["q"]
+        got = _gpu(pkg, dev, q, cut, canary=True)
+        _gate(got, orc.fmha_i8_blockwise_cross(q, cut["k"], cut["v"], cut["mask"], *_scales(c)),
+              "S=%d Sq=%d d=%d" % (S, Sq, d))
+        # (not bit for bit: the last block's keys sit in other lanes than in the padded run, so the float row sum
+        # adds them in another order)
+        st = fc.parity_stats(got, _gpu(pkg, dev, q, padded))
+        assert st["max"] <= 1 and st["exact"] >= 0.999, (S, Sq, st)
+
+
+@pytest.mark.gpu
+def test_any_key_count_at_the_end_of_an_allocation(pkg, orc, dev):
+    """K, V and the mask end exactly where their device allocations end: a tile load or a mask read that ran past the
+    last key would leave the buffers (the last head of the last batch entry is the one that matters)."""
+    import torch
+    B, H, S, d = 1, 2, 70, 128
+    c = fc.make_inputs(B, H, 128, d, seed=63)
+    k, v, m = (np.ascontiguousarray(a) for a in (c["k"][:, :, :S], c["v"][:, :, :S], c["mask"][:, :S]))
+    q = c["q"][:, :, :40]
+    want = orc.fmha_i8_blockwise_cross(q, k, v, m, *_scales(c))
+    bufs = []
+    for a in (k, v, m):
+        n = a.size
+        buf = torch.empty(((n + 4095) // 4096) * 4096, dtype=torch.int8, device=dev)
+        view = buf[buf.numel() - n:].view(a.shape) if n % 16 == 0 else None
+        if view is None:  # the mask has no alignment requirement: put it at the very end, whatever its size
+            view = buf[buf.numel() - n:].view(a.shape)
+        view.copy_(torch.from_numpy(a))
+        bufs.append((buf, view))
+    qd = torch.from_numpy(np.ascontiguousarray(q)).to(dev)
+    o = pkg.fmha_infer_i8(qd, bufs[0][1], bufs[1][1], bufs[2][1], *_scales(c))
+    torch.cuda.synchronize()
+    _gate(o.cpu().numpy(), want, "end of allocation")

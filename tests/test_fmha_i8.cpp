@@ -248,7 +248,7 @@ bool run_case(const Case& c, const Options& opt, FILE* json) {
     auto t0 = std::chrono::steady_clock::now();
     fmha_oracle::fmha_i8_cpu_blockwise_cross(t.q.data(), t.k.data(), t.v.data(), t.mask.data(), want.data(), c.B, c.H,
                                              Sq, c.S, c.d, t.q_amax, t.k_amax, t.v_amax, o_amax,
-                                             c.S % 128 == 0 ? 128 : 64, threads, 0, cpu_heads);
+                                             (c.S + 63) / 64 * 64 % 128 == 0 ? 128 : 64, threads, 0, cpu_heads);
     cpu_i8_s = seconds_since(t0);
     const long m = cpu_heads * Sq * c.d;
     int worst = 0;

@@ -64,10 +64,11 @@ def test_argument_checks_need_no_gpu(pkg):
     for d in (0, 32, 96, 256):
         assert pkg.FMHAInferI8CheckArgs(P, pkg.AttnDataDescriptor(1, 128, 1, d), a16, a16, a16, a16, a16) == \
             pkg.FMHA_I8_ERR_HEAD_DIM
-    for s in (0, -128, 32, 100, 1000, 65600):
+    for s in (0, -128, 65537, 65600):
         assert pkg.FMHAInferI8CheckArgs(P, pkg.AttnDataDescriptor(1, s, 1, 64), a16, a16, a16, a16, a16) == \
             pkg.FMHA_I8_ERR_SEQ_LEN
-    for s in (64, 128, 192, 320, 448, 512, 4096, 65536):  # every length of the reference's ladder (src/fmha_i8.cu:39-154)
+    # every length of the reference's ladder (src/fmha_i8.cu:39-154), and lengths it does not have
+    for s in (64, 128, 192, 320, 448, 512, 4096, 65536, 1, 32, 100, 1000):
         assert pkg.FMHAInferI8CheckArgs(P, pkg.AttnDataDescriptor(1, s, 1, 64), a16, a16, a16, a16, a16) == pkg.FMHA_I8_OK
     assert pkg.FMHAInferI8CheckArgs(P, pkg.AttnDataDescriptor(0, 128, 1, 64), a16, a16, a16, a16, a16) == \
         pkg.FMHA_I8_ERR_BATCH_HEAD

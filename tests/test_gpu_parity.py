@@ -371,13 +371,13 @@ def test_unsupported_shapes_leave_output_untouched(pkg, dev):
     m = torch.zeros(1, 160, dtype=torch.int8, device=dev)
     o = torch.full_like(q, 55)
     P = pkg.FMHAParamI8(1, 1, 1, 1)
-    assert pkg.FMHAInferI8Status(None, P, pkg.AttnDataDescriptor(1, 160, 1, 64), q, q, q, m, o) == \
+    assert pkg.FMHAInferI8Status(None, P, pkg.AttnDataDescriptor(1, 65537, 1, 64), q, q, q, m, o) == \
         pkg.FMHA_I8_ERR_SEQ_LEN
     pkg.FMHAInferI8(None, P, pkg.AttnDataDescriptor(1, 128, 1, 96), q, q, q, m, o, True)  # prints, launches nothing
     torch.cuda.synchronize()
     assert bool((o == 55).all())
     with pytest.raises(pkg.FMHAError):
-        pkg.fmha_infer_i8(q, q, q, m, 1.0, 1.0, 1.0)
+        pkg.fmha_infer_i8(q, q, q, m, 1.0, 1.0, 1.0, o_amax=0.0)
 
 
 # ---- the C++ harness (host C++ calling the C ABI the way the reference's driver calls its launch function) -------------
