@@ -246,16 +246,19 @@ def test_saturation_and_clamp(pkg, orc, dev):
     check(gpu_run(pkg, dev, c, v_amax=4 * c["v_amax"]), want, "saturating")
 
 
-@pytest.mark.parametrize("S,d", [(512, 128), (512, 64), (320, 128), (320, 64)])
+@pytest.mark.parametrize("S,d", [(512, 128), (512, 64), (320, 128), (320, 64), (500, 128), (500, 64), (300, 128), (300, 64)])
 @pytest.mark.parametrize("qk_scale,vo_ratio", [(1.0, 1.0), (1.0, 60.0), (40.0, 1.0), (40.0, 60.0)])
 def test_every_kernel_variant(pkg, orc, dev, S, d, qk_scale, vo_ratio):
     """The library picks one of four arithmetic variants of the kernel from the scales (accumulators read as floats or
-    converted; accumulator offset folded into the running O or not) for each head_dim and softmax block size.  A large
-    q_amax*k_amax forces the converting variant, a large v_amax/o_amax the unfolded one: all sixteen instantiations
-    must meet the same gate."""
+    converted; accumulator offset folded into the running O or not) for each head_dim, softmax block size (128 or 64
+    keys) and for lengths with and without a partly filled last block.  A large q_amax*k_amax forces the converting
+    variant, a large v_amax/o_amax the unfolded one: all thirty-two instantiations must meet the same gate."""
     c = fc.make_inputs(2, 2, S, d, dist="normal", pad="scatter", seed=91)
     kw = dict(q_amax=c["q_amax"] * qk_scale, v_amax=vo_ratio, o_amax=1.0 if vo_ratio == 1.0 else 2.0)
-    check(gpu_run(pkg, dev, c, **kw), cpu_run(orc, c, **kw), "variant S=%d d=%d qk=%g vo=%g" % (S, d, qk_scale, vo_ratio))
+    s = dict(q_amax=c["q_amax"], k_amax=c["k_amax"], v_amax=c["v_amax"], o_amax=c["o_amax"])
+    s.update(kw)
+    want = orc.fmha_i8_blockwise_cross(c["q"], c["k"], c["v"], c["mask"], s["q_amax"], s["k_amax"], s["v_amax"], s["o_amax"])
+    check(gpu_run(pkg, dev, c, **kw), want, "variant S=%d d=%d qk=%g vo=%g" % (S, d, qk_scale, vo_ratio))
 
 
 @pytest.mark.parametrize("S,d", [(256, 128), (192, 64)])
