@@ -307,13 +307,17 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     }
   }
   // last key block that holds any unmasked key (trailing padding is never computed on)
-  int last_block = -1;
+  int last_block = -1, first_padded = n_blocks;  // (and the first block with any masked key)
   for (int base = 0; base < n_blocks; base += 64) {
     const int blk = base + lane;
-    const unsigned long long live = __ballot(blk < n_blocks && !(lds_class[blk < n_blocks ? blk : 0] & 2));
+    const int c = lds_class[blk < n_blocks ? blk : 0];
+    const unsigned long long live = __ballot(blk < n_blocks && !(c & 2));
+    const unsigned long long padded = __ballot(blk < n_blocks && c != 0);
     if (live != 0) last_block = base + 63 - __builtin_clzll(live);
+    if (padded != 0 && first_padded == n_blocks) first_padded = base + __builtin_ctzll(padded);
   }
   const int kb_end = __builtin_amdgcn_readfirstlane(last_block) + 1;
+  const int kb_plain = __builtin_amdgcn_readfirstlane(first_padded);  // blocks [0, kb_plain) have no masked key
 
   float o_f[kDSteps][16];
 #pragma unroll
@@ -559,22 +563,25 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   const int n = kb_end;
   auto cls_of = [&](int kb) { return __builtin_amdgcn_readfirstlane((int)lds_class[kb]); };
   auto works = [&](int kb) { return active && !(cls_of(kb) & 2); };  // nothing in a fully masked block is attended to
+  // Every issue point issues the same number of tiles whatever the position in the sequence: a tile index past the
+  // last block is replaced by the last block, which is then fetched again into the stage it already occupies (the
+  // same bytes: harmless for the wavefronts reading it).  That keeps the wait counts below compile-time constants and
+  // the key loop free of the compares and branches that a count depending on the position would need.
+  const int last = n - 1;
   auto issue_first = [&]() {          // after barrier 0
-    if (n > 1) issue_k(1);
-    if (n > 2) issue_k(2);
-    if (n > 1) issue_v(1);
+    if (n > 0) {
+      issue_k(min(1, last));
+      issue_k(min(2, last));
+      issue_v(min(1, last));
+    }
   };
   auto issue_after_softmax = [&](int i) {
-    if (i + 3 < n) issue_k(i + 3);
-    if (i + 2 < n) issue_v(i + 2);
+    issue_k(min(i + 3, last));
+    issue_v(min(i + 2, last));
   };
   // Before barrier 2m every wavefront waits for its share of K(m) and V(m-1).  Tiles issued later may stay in flight:
   // K(m+1), V(m) (after Y(m-2)) and, for the wavefronts that have already finished Y(m-1), K(m+2), V(m+1).
-  auto wait_tiles_for = [&](int m, bool after_next_softmax) {
-    int newer = (m + 1 < n ? 1 : 0) + (m < n ? 1 : 0);
-    if (after_next_softmax) newer += (m + 2 < n ? 1 : 0) + (m + 1 < n ? 1 : 0);
-    wait_all_but(newer);
-  };
+  auto wait_tiles_for = [&](bool after_next_softmax) { wait_all_but(after_next_softmax ? 4 : 2); };
   v16i acc[kKeyTiles];  // S^T of the block whose softmax comes next (GEMM 1 -> softmax, across a barrier)
   int mx[2];
   // Where GEMM 1 is skipped the old scores are dead; saying so (an empty definition) keeps 64 registers from being
@@ -593,14 +600,32 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     if (n > 0 && works(0)) phase_gemm1(0, acc, mx);
     else forget_scores();
     issue_first();
-    for (int i = 0; i < n; ++i) {
+    int i = 0;
+    // Steady state, as long as blocks i and i+1 exist and have no masked key: the same phases as the general loop
+    // below with every decision taken (scalar compares and branches are not free: they stand in the issue stream of
+    // the wavefront that the barrier is waiting for).
+    if (active) {
+      for (; i + 1 < n && i + 1 < kb_plain; ++i) {
+        v4i pk[kKeyTiles];
+        barrier();
+        phase_softmax(i, 0, acc, pk, mx);
+        issue_after_softmax(i);
+        wait_tiles_for(true);
+        barrier();
+        raise_priority();
+        phase_gemm2_merge(i, pk);
+        phase_gemm1(i + 1, acc, mx);
+        drop_priority();
+      }
+    }
+    for (; i < n; ++i) {
       const int cls = cls_of(i);
       const bool work = active && !(cls & 2);
       v4i pk[kKeyTiles];
       barrier();                               // barrier 2i+1
       if (work) phase_softmax(i, cls, acc, pk, mx);
       issue_after_softmax(i);
-      wait_tiles_for(i + 1, true);
+      wait_tiles_for(true);
       barrier();                               // barrier 2i+2
       raise_priority();
       if (work) phase_gemm2_merge(i, pk);
@@ -614,11 +639,26 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     barrier();                                 // barrier 1
     if (n > 0 && works(0)) phase_gemm1(0, acc, mx);
     else forget_scores();
-    for (int i = 0; i < n; ++i) {
+    int i = 0;
+    if (active) {  // steady state, see above
+      for (; i + 1 < n && i + 1 < kb_plain; ++i) {
+        v4i pk[kKeyTiles];
+        wait_tiles_for(false);
+        barrier();
+        phase_softmax(i, 0, acc, pk, mx);
+        issue_after_softmax(i);
+        barrier();
+        raise_priority();
+        phase_gemm2_merge(i, pk);
+        phase_gemm1(i + 1, acc, mx);
+        drop_priority();
+      }
+    }
+    for (; i < n; ++i) {
       const int cls = cls_of(i);
       const bool work = active && !(cls & 2);
       v4i pk[kKeyTiles];
-      wait_tiles_for(i + 1, false);
+      wait_tiles_for(false);
       barrier();                               // barrier 2i+2
       if (work) phase_softmax(i, cls, acc, pk, mx);
       issue_after_softmax(i);
