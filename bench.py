@@ -31,7 +31,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 INT8_PEAK_TOPS = 5033.2  # 256 CU * 8192 op/clk/CU * 2.4 GHz
 # HBM bytes per launch of the headline workload measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by
 # what the same counter reads for a plain copy kernel of known size): 25.46 MB read + 8.39 MB written.
-MEASURED_TRAFFIC_BYTES = {"C3": 33.85e6}
+MEASURED_TRAFFIC_BYTES = {"C3": 33.92e6}
 
 
 def cpu_baseline(orc, c, sample_heads, threads):
