@@ -35,6 +35,15 @@ int FMHAQuantizeI8(hipStream_t stream, const float* x, long long n, float amax_h
 /* The de-quantisation the reference prints and scores with (inc/utils.hpp:53,70): out[i] = (float)x[i] / 127 * amax. */
 int FMHADequantizeI8(hipStream_t stream, const int8_t* x, long long n, float amax, float* out);
 
+/* The same three steps for bfloat16 tensors (raw 16-bit patterns; torch.bfloat16 storage).  A bfloat16 widens to a
+ * float exactly, so the results are those of the float functions above applied to the widened values; the de-quantised
+ * value is rounded to bfloat16 once, to nearest even.  (The reference's driver only has float tensors,
+ * test_fmha_i8.cpp:58-62; a bfloat16 producer would otherwise pay a widening pass over HBM first.) */
+int FMHAAbsMaxBF16(hipStream_t stream, const uint16_t* x, long long n, float* amax_out);
+int FMHAQuantizeI8BF16(hipStream_t stream, const uint16_t* x, long long n, float amax_host, const float* amax_dev,
+                       int8_t* out);
+int FMHADequantizeI8BF16(hipStream_t stream, const int8_t* x, long long n, float amax, uint16_t* out);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif

@@ -17,7 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libfmha_i8.so")
 
 EXPORTED_SYMBOLS = ("FMHAInferI8", "FMHAInferI8Status", "FMHAInferI8CheckArgs", "FMHAInferI8StatusString",
                     "FMHAInferI8Version", "FMHAInferI8Cross", "FMHAInferI8CrossCheckArgs", "FMHAAbsMaxF32",
-                    "FMHAQuantizeI8", "FMHADequantizeI8")
+                    "FMHAQuantizeI8", "FMHADequantizeI8", "FMHAAbsMaxBF16", "FMHAQuantizeI8BF16", "FMHADequantizeI8BF16")
 
 FMHA_I8_OK = 0
 FMHA_I8_ERR_NULL_POINTER = 1
@@ -101,6 +101,12 @@ def load_library(path=None):
     L.FMHAQuantizeI8.restype = C.c_int
     L.FMHADequantizeI8.argtypes = [ptr, ptr, C.c_longlong, C.c_float, ptr]
     L.FMHADequantizeI8.restype = C.c_int
+    L.FMHAAbsMaxBF16.argtypes = L.FMHAAbsMaxF32.argtypes
+    L.FMHAAbsMaxBF16.restype = C.c_int
+    L.FMHAQuantizeI8BF16.argtypes = L.FMHAQuantizeI8.argtypes
+    L.FMHAQuantizeI8BF16.restype = C.c_int
+    L.FMHADequantizeI8BF16.argtypes = L.FMHADequantizeI8.argtypes
+    L.FMHADequantizeI8BF16.restype = C.c_int
     if path is None:
         _lib = L
     return L
@@ -178,32 +184,51 @@ def FMHADequantizeI8(stream, x, n, amax, out):
     return int(load_library().FMHADequantizeI8(_stream(stream), _ptr(x), int(n), float(amax), _ptr(out)))
 
 
+def FMHAAbsMaxBF16(stream, x, n, amax_out):
+    """FMHAAbsMaxF32 for a bfloat16 tensor (raw 16-bit patterns)."""
+    return int(load_library().FMHAAbsMaxBF16(_stream(stream), _ptr(x), int(n), _ptr(amax_out)))
+
+
+def FMHAQuantizeI8BF16(stream, x, n, amax_host, amax_dev, out):
+    """FMHAQuantizeI8 for a bfloat16 tensor: same roundings as on the widened floats."""
+    return int(load_library().FMHAQuantizeI8BF16(_stream(stream), _ptr(x), int(n), float(amax_host), _ptr(amax_dev), _ptr(out)))
+
+
+def FMHADequantizeI8BF16(stream, x, n, amax, out):
+    """FMHADequantizeI8 with the result rounded to bfloat16 (nearest even)."""
+    return int(load_library().FMHADequantizeI8BF16(_stream(stream), _ptr(x), int(n), float(amax), _ptr(out)))
+
+
 def quantize_tensor(x, amax=None, stream=None):
-    """Convenience for a contiguous fp32 torch tensor on the GPU: returns (int8 tensor, amax as a 1-element device
-    tensor).  With amax=None the maximum is measured on the GPU and never visits the host."""
+    """Convenience for a contiguous float32 or bfloat16 torch tensor on the GPU: returns (int8 tensor, amax as a
+    1-element float32 device tensor).  With amax=None the maximum is measured on the GPU and never visits the host."""
     import torch
-    if not (x.is_cuda and x.dtype == torch.float32 and x.is_contiguous()):
-        raise ValueError("x must be a contiguous float32 tensor on the GPU")
+    if not (x.is_cuda and x.dtype in (torch.float32, torch.bfloat16) and x.is_contiguous()):
+        raise ValueError("x must be a contiguous float32 or bfloat16 tensor on the GPU")
+    absmax, quant = (FMHAAbsMaxF32, FMHAQuantizeI8) if x.dtype == torch.float32 else (FMHAAbsMaxBF16, FMHAQuantizeI8BF16)
     st = stream if stream is not None else torch.cuda.current_stream(x.device)
     out = torch.empty(x.shape, dtype=torch.int8, device=x.device)
     if amax is None:
         a = torch.empty(1, dtype=torch.float32, device=x.device)
-        _check(FMHAAbsMaxF32(st, x, x.numel(), a))
-        _check(FMHAQuantizeI8(st, x, x.numel(), 0.0, a, out))
+        _check(absmax(st, x, x.numel(), a))
+        _check(quant(st, x, x.numel(), 0.0, a, out))
     else:
         a = torch.full((1,), float(amax), dtype=torch.float32, device=x.device)
-        _check(FMHAQuantizeI8(st, x, x.numel(), float(amax), None, out))
+        _check(quant(st, x, x.numel(), float(amax), None, out))
     return out, a
 
 
-def dequantize_tensor(x, amax, stream=None):
-    """int8 torch tensor on the GPU -> float32, (float)x / 127 * amax."""
+def dequantize_tensor(x, amax, stream=None, dtype=None):
+    """int8 torch tensor on the GPU -> float32 (default) or bfloat16, (float)x / 127 * amax."""
     import torch
     if not (x.is_cuda and x.dtype == torch.int8 and x.is_contiguous()):
         raise ValueError("x must be a contiguous int8 tensor on the GPU")
+    dtype = dtype or torch.float32
+    if dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("dtype must be float32 or bfloat16")
     st = stream if stream is not None else torch.cuda.current_stream(x.device)
-    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
-    _check(FMHADequantizeI8(st, x, x.numel(), float(amax), out))
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    _check((FMHADequantizeI8 if dtype == torch.float32 else FMHADequantizeI8BF16)(st, x, x.numel(), float(amax), out))
     return out
 
 

@@ -107,7 +107,17 @@ __global__ __launch_bounds__(kQuantThreads) void quantize_i8_kernel(const float*
     out[4 * units + threadIdx.x] = (int8_t)quant1_nan0(x[4 * units + threadIdx.x], scale);
 }
 
-// inc/utils.hpp:53: (float)v / 127.0f * amax, in that order.
+// inc/utils.hpp:53: (float)v / 127.0f * amax, in that order.  The quotient is formed without the division sequence:
+// q0 = v * fl(1/127), the exact remainder r = v - 127 q0 (one fma), q = q0 + r * fl(1/127) (one fma).  For each of the
+// 256 values of v this is the correctly rounded v / 127.0f (checked exhaustively by the tests); a quarter of the
+// instructions, and these kernels have to keep up with HBM.
+__device__ __forceinline__ float dequant1(int v, float amax) {
+  constexpr float kRcp127 = 1.0f / 127.0f;
+  const float fv = (float)v;
+  const float q0 = fv * kRcp127;
+  const float r = __builtin_fmaf(-q0, 127.0f, fv);
+  return __builtin_fmaf(r, kRcp127, q0) * amax;
+}
 template <bool NT>
 __global__ __launch_bounds__(kQuantThreads) void dequantize_i8_kernel(const int8_t* __restrict__ x, long long n,
                                                                        float amax, float* __restrict__ out) {
@@ -115,7 +125,7 @@ __global__ __launch_bounds__(kQuantThreads) void dequantize_i8_kernel(const int8
   const int* __restrict__ x4 = reinterpret_cast<const int*>(x);
   v4f* __restrict__ o4 = reinterpret_cast<v4f*>(out);
   const long long stride = (long long)gridDim.x * kQuantThreads;
-  auto one = [&](int v) { return (float)v / 127.0f * amax; };
+  auto one = [&](int v) { return dequant1(v, amax); };
   auto unpack = [&](int w) {
     return v4f{one((int8_t)(w & 0xff)), one((int8_t)((w >> 8) & 0xff)), one((int8_t)((w >> 16) & 0xff)), one(w >> 24)};
   };
@@ -132,6 +142,122 @@ __global__ __launch_bounds__(kQuantThreads) void dequantize_i8_kernel(const int8
   }
   for (; j < units; j += stride) o4[j] = unpack(x4[j]);
   if (blockIdx.x == 0 && threadIdx.x < (int)(n - 4 * units)) out[4 * units + threadIdx.x] = one(x[4 * units + threadIdx.x]);
+}
+
+// ---- bfloat16 tensors ---------------------------------------------------------------------------------------------
+// A bfloat16 is the upper half of a float: widening is exact, so the three functions below are the float ones applied
+// to the widened values (same roundings, same results); the de-quantised float is rounded to bfloat16 once, to nearest
+// even.  One 16-byte unit holds eight elements.
+typedef unsigned short v8h __attribute__((ext_vector_type(8)));
+typedef unsigned short v4h __attribute__((ext_vector_type(4)));
+typedef int v2i32 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float widen(unsigned short h) { return __uint_as_float((unsigned)h << 16); }
+__device__ __forceinline__ unsigned short narrow_rne(float f) {
+  const unsigned u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40u);  // NaN stays NaN
+  return (unsigned short)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+__global__ __launch_bounds__(kQuantThreads) void abs_max_bf16_kernel(const unsigned short* __restrict__ x, long long n,
+                                                                      float* __restrict__ out) {
+  const long long units = n / 8;
+  const v8h* __restrict__ x8 = reinterpret_cast<const v8h*>(x);
+  const long long stride = (long long)gridDim.x * kQuantThreads;
+  float m = 0.f;
+  auto take = [&](unsigned short h) {
+    const float a = fabsf(widen(h));
+    m = a > m ? a : m;  // a NaN never compares greater: skipped
+  };
+  long long j = (long long)blockIdx.x * kQuantThreads + threadIdx.x;
+  for (; j + (kQuantUnroll - 1) * stride < units; j += kQuantUnroll * stride) {
+    v8h v[kQuantUnroll];
+#pragma unroll
+    for (int u = 0; u < kQuantUnroll; ++u) v[u] = x8[j + u * stride];
+#pragma unroll
+    for (int u = 0; u < kQuantUnroll; ++u)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) take(v[u][e]);
+  }
+  for (; j < units; j += stride) {
+    const v8h v = x8[j];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) take(v[e]);
+  }
+  if (blockIdx.x == 0 && threadIdx.x < (int)(n - 8 * units)) take(x[8 * units + threadIdx.x]);
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float o = __shfl_xor(m, off);
+    m = o > m ? o : m;
+  }
+  __shared__ float part[kQuantThreads / 64];
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int w = 1; w < kQuantThreads / 64; ++w) m = part[w] > m ? part[w] : m;
+    if (m > 0.f) atomicMax(reinterpret_cast<unsigned int*>(out), __float_as_uint(m));
+  }
+}
+
+template <bool NT>
+__global__ __launch_bounds__(kQuantThreads) void quantize_i8_bf16_kernel(const unsigned short* __restrict__ x, long long n,
+                                                                          float amax_host,
+                                                                          const float* __restrict__ amax_dev,
+                                                                          int8_t* __restrict__ out) {
+  const float amax = amax_dev != nullptr ? *amax_dev : amax_host;
+  const float scale = 127.0f / amax;
+  const long long units = n / 8;
+  const v8h* __restrict__ x8 = reinterpret_cast<const v8h*>(x);
+  v2i32* __restrict__ o8 = reinterpret_cast<v2i32*>(out);
+  const long long stride = (long long)gridDim.x * kQuantThreads;
+  auto q = [&](unsigned short h) { return quant1_nan0(widen(h), scale) & 0xff; };
+  auto pack = [&](const v8h& v) {
+    return v2i32{q(v[0]) | (q(v[1]) << 8) | (q(v[2]) << 16) | (q(v[3]) << 24),
+                 q(v[4]) | (q(v[5]) << 8) | (q(v[6]) << 16) | (q(v[7]) << 24)};
+  };
+  long long j = (long long)blockIdx.x * kQuantThreads + threadIdx.x;
+  for (; j + (kQuantUnroll - 1) * stride < units; j += kQuantUnroll * stride) {
+    v8h v[kQuantUnroll];
+#pragma unroll
+    for (int u = 0; u < kQuantUnroll; ++u) v[u] = NT ? __builtin_nontemporal_load(&x8[j + u * stride]) : x8[j + u * stride];
+#pragma unroll
+    for (int u = 0; u < kQuantUnroll; ++u) {
+      if (NT) __builtin_nontemporal_store(pack(v[u]), &o8[j + u * stride]);
+      else o8[j + u * stride] = pack(v[u]);
+    }
+  }
+  for (; j < units; j += stride) o8[j] = pack(x8[j]);
+  if (blockIdx.x == 0 && threadIdx.x < (int)(n - 8 * units))
+    out[8 * units + threadIdx.x] = (int8_t)quant1_nan0(widen(x[8 * units + threadIdx.x]), scale);
+}
+
+template <bool NT>
+__global__ __launch_bounds__(kQuantThreads) void dequantize_i8_bf16_kernel(const int8_t* __restrict__ x, long long n,
+                                                                            float amax, unsigned short* __restrict__ out) {
+  const long long units = n / 8;
+  const v2i32* __restrict__ x8 = reinterpret_cast<const v2i32*>(x);
+  v8h* __restrict__ o8 = reinterpret_cast<v8h*>(out);
+  const long long stride = (long long)gridDim.x * kQuantThreads;
+  auto one = [&](int v) { return narrow_rne(dequant1(v, amax)); };
+  auto unpack = [&](const v2i32& w) {
+    v8h r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = one((int8_t)((w[e >> 2] >> (8 * (e & 3))) & 0xff));
+    return r;
+  };
+  long long j = (long long)blockIdx.x * kQuantThreads + threadIdx.x;
+  for (; j + (kQuantUnroll - 1) * stride < units; j += kQuantUnroll * stride) {
+    v2i32 w[kQuantUnroll];
+#pragma unroll
+    for (int u = 0; u < kQuantUnroll; ++u) w[u] = NT ? __builtin_nontemporal_load(&x8[j + u * stride]) : x8[j + u * stride];
+#pragma unroll
+    for (int u = 0; u < kQuantUnroll; ++u) {
+      if (NT) __builtin_nontemporal_store(unpack(w[u]), &o8[j + u * stride]);
+      else o8[j + u * stride] = unpack(w[u]);
+    }
+  }
+  for (; j < units; j += stride) o8[j] = unpack(x8[j]);
+  if (blockIdx.x == 0 && threadIdx.x < (int)(n - 8 * units)) out[8 * units + threadIdx.x] = one(x[8 * units + threadIdx.x]);
 }
 
 inline int quant_blocks(long long n) {
@@ -181,6 +307,44 @@ int FMHADequantizeI8(hipStream_t stream, const int8_t* x, long long n, float ama
     hipLaunchKernelGGL(dequantize_i8_kernel<true>, dim3(quant_blocks(n)), dim3(kQuantThreads), 0, stream, x, n, amax, out);
   else
     hipLaunchKernelGGL(dequantize_i8_kernel<false>, dim3(quant_blocks(n)), dim3(kQuantThreads), 0, stream, x, n, amax, out);
+  return launch_status();
+}
+
+int FMHAAbsMaxBF16(hipStream_t stream, const uint16_t* x, long long n, float* amax_out) {
+  using namespace fmha_i8_gfx950;
+  if (amax_out == nullptr || (x == nullptr && n > 0) || n < 0) return FMHA_I8_ERR_NULL_POINTER;
+  if (!aligned16(x)) return FMHA_I8_ERR_ALIGNMENT;
+  hipLaunchKernelGGL(zero_float_kernel, dim3(1), dim3(1), 0, stream, amax_out);
+  if (n > 0)
+    hipLaunchKernelGGL(abs_max_bf16_kernel, dim3(quant_blocks(n / 2)), dim3(kQuantThreads), 0, stream, x, n, amax_out);
+  return launch_status();
+}
+
+int FMHAQuantizeI8BF16(hipStream_t stream, const uint16_t* x, long long n, float amax_host, const float* amax_dev,
+                       int8_t* out) {
+  using namespace fmha_i8_gfx950;
+  if (n < 0 || ((x == nullptr || out == nullptr) && n > 0)) return FMHA_I8_ERR_NULL_POINTER;
+  if (!aligned16(x) || !aligned16(out)) return FMHA_I8_ERR_ALIGNMENT;
+  if (amax_dev == nullptr && !(amax_host == amax_host)) return FMHA_I8_ERR_SCALE;
+  if (n == 0) return FMHA_I8_OK;
+  if (3 * n > kCacheBytes)
+    hipLaunchKernelGGL(quantize_i8_bf16_kernel<true>, dim3(quant_blocks(n / 2)), dim3(kQuantThreads), 0, stream, x, n,
+                       amax_host, amax_dev, out);
+  else
+    hipLaunchKernelGGL(quantize_i8_bf16_kernel<false>, dim3(quant_blocks(n / 2)), dim3(kQuantThreads), 0, stream, x, n,
+                       amax_host, amax_dev, out);
+  return launch_status();
+}
+
+int FMHADequantizeI8BF16(hipStream_t stream, const int8_t* x, long long n, float amax, uint16_t* out) {
+  using namespace fmha_i8_gfx950;
+  if (n < 0 || ((x == nullptr || out == nullptr) && n > 0)) return FMHA_I8_ERR_NULL_POINTER;
+  if (!aligned16(x) || !aligned16(out)) return FMHA_I8_ERR_ALIGNMENT;
+  if (n == 0) return FMHA_I8_OK;
+  if (3 * n > kCacheBytes)
+    hipLaunchKernelGGL(dequantize_i8_bf16_kernel<true>, dim3(quant_blocks(n / 2)), dim3(kQuantThreads), 0, stream, x, n, amax, out);
+  else
+    hipLaunchKernelGGL(dequantize_i8_bf16_kernel<false>, dim3(quant_blocks(n / 2)), dim3(kQuantThreads), 0, stream, x, n, amax, out);
   return launch_status();
 }
 

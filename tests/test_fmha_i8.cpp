@@ -336,9 +336,48 @@ static bool run_quant(long mib, const Options& opt) {
     if (q[(size_t)i] != (int8_t)fmha_oracle::quantize_i8(x[(size_t)i], want_amax)) ++bad_q;
     if (back[(size_t)i] != (float)q[(size_t)i] / 127.0f * 17.25f) ++bad_d;
   }
-  const bool ok = amax == want_amax && bad_q == 0 && bad_d == 0;
+  bool ok = amax == want_amax && bad_q == 0 && bad_d == 0;
   printf("quantisation parity over %lld elements: amax %g (checker %g), quantise mismatches %lld, de-quantise mismatches "
          "%lld  [%s]\n", n, amax, want_amax, bad_q, bad_d, ok ? "PASS" : "FAIL");
+
+  // the same element count as bfloat16 (the upper halves of the floats above): checked against the widened values
+  std::vector<uint16_t> h((size_t)n);
+  std::vector<float> wide((size_t)n);
+  for (long long i = 0; i < n; ++i) {
+    uint32_t u;
+    memcpy(&u, &x[(size_t)i], 4);
+    h[(size_t)i] = (uint16_t)(u >> 16);
+    u &= 0xffff0000u;
+    memcpy(&wide[(size_t)i], &u, 4);
+  }
+  uint16_t* dh = reinterpret_cast<uint16_t*>(dx);        // reuse the float buffers: half the bytes
+  uint16_t* dhback = reinterpret_cast<uint16_t*>(dback);
+  CHECK_HIP(hipMemcpy(dh, h.data(), (size_t)n * 2, hipMemcpyHostToDevice));
+  st = 0;
+  timed("FMHAAbsMaxBF16", 2.0 * n, [&] { st |= FMHAAbsMaxBF16(stream, dh, n, dam); });
+  timed("FMHAQuantizeI8BF16 (device amax)", 3.0 * n, [&] { st |= FMHAQuantizeI8BF16(stream, dh, n, 0.f, dam, dq); });
+  timed("FMHADequantizeI8BF16", 3.0 * n, [&] { st |= FMHADequantizeI8BF16(stream, dq, n, 17.25f, dhback); });
+  if (st != FMHA_I8_OK) {
+    fprintf(stderr, "bfloat16 quantisation entry points failed: %s\n", FMHAInferI8StatusString(st));
+    return false;
+  }
+  std::vector<uint16_t> hback((size_t)n);
+  CHECK_HIP(hipMemcpy(&amax, dam, 4, hipMemcpyDeviceToHost));
+  CHECK_HIP(hipMemcpy(q.data(), dq, (size_t)n, hipMemcpyDeviceToHost));
+  CHECK_HIP(hipMemcpy(hback.data(), dhback, (size_t)n * 2, hipMemcpyDeviceToHost));
+  const float want_amax_h = fmha_oracle::abs_max(wide.data(), n);
+  bad_q = bad_d = 0;
+  for (long long i = 0; i < n; ++i) {
+    if (q[(size_t)i] != (int8_t)fmha_oracle::quantize_i8(wide[(size_t)i], want_amax_h)) ++bad_q;
+    const float f = (float)q[(size_t)i] / 127.0f * 17.25f;
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if (hback[(size_t)i] != (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16)) ++bad_d;
+  }
+  const bool ok_h = amax == want_amax_h && bad_q == 0 && bad_d == 0;
+  printf("bfloat16 quantisation parity over %lld elements: amax %g (checker %g), quantise mismatches %lld, de-quantise "
+         "mismatches %lld  [%s]\n", n, amax, want_amax_h, bad_q, bad_d, ok_h ? "PASS" : "FAIL");
+  ok = ok && ok_h;
   CHECK_HIP(hipFree(dx)), CHECK_HIP(hipFree(dback)), CHECK_HIP(hipFree(dq)), CHECK_HIP(hipFree(dam));
   return ok;
 }

@@ -124,3 +124,57 @@ def test_float_tensors_through_the_whole_path(pkg, orc, dev):
     st = fc.parity_stats(o8.cpu().numpy(), want8)
     assert st["within1"] >= 0.999 and st["max"] <= 2, st
     assert np.array_equal(of.cpu().numpy(), o8.cpu().numpy().astype(np.float32) / np.float32(127.0) * np.float32(1.0))
+
+
+# ---- bfloat16 tensors --------------------------------------------------------------------------------------------
+def _to_bf16_bits(x):
+    """float32 -> bfloat16 bit patterns, round to nearest even (finite inputs)."""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def _widen(bits):
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+@pytest.mark.parametrize("n", [0, 1, 7, 8, 9, 31, 4096, 1000003])
+def test_bf16_abs_max_and_quantize_match_the_checker_on_the_widened_values(pkg, orc, dev, n):
+    import torch
+    rng = np.random.default_rng(300 + n)
+    bits = _to_bf16_bits(3.0 * rng.standard_normal(n))
+    wide = _widen(bits)
+    xd = torch.from_numpy(bits.view(np.int16)).to(dev).view(torch.bfloat16)
+    q, a = pkg.quantize_tensor(xd)
+    torch.cuda.synchronize()
+    amax = float(np.abs(wide).max()) if n else 0.0
+    assert a.item() == np.float32(amax)
+    if n:
+        assert np.array_equal(q.cpu().numpy(), orc.quantize_i8(wide, amax))
+        # and with the scale passed by value, ties and clamps included
+        bits2 = _to_bf16_bits(np.array([0.5, -0.5, 1.5, 2.5, -2.5, 126.5, 127.0, 200.0, -200.0, 0.49609375], np.float32))
+        x2 = torch.from_numpy(bits2.view(np.int16)).to(dev).view(torch.bfloat16)
+        q2, _ = pkg.quantize_tensor(x2, amax=127.0)
+        assert np.array_equal(q2.cpu().numpy(), orc.quantize_i8(_widen(bits2), 127.0))
+
+
+@pytest.mark.parametrize("n", [0, 1, 9, 4096, 300001])
+def test_bf16_dequantize_rounds_the_float_result_once(pkg, dev, n):
+    import torch
+    v = np.random.default_rng(400 + n).integers(-128, 128, n).astype(np.int8)
+    amax = 3.3
+    out = pkg.dequantize_tensor(_dev(dev, v), amax, dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+    want = _to_bf16_bits(v.astype(np.float32) / np.float32(127.0) * np.float32(amax))
+    assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), want)
+
+
+def test_bf16_nan_is_skipped_and_quantises_to_zero(pkg, dev):
+    import torch
+    bits = np.array([0x7FC0, 0x3F80, 0xFFC1, 0xC000, 0x0000, 0x8000, 0x3F00, 0x4000, 0x7F80], np.uint16)  # NaN 1 NaN -2 0 -0 .5 2 inf
+    xd = torch.from_numpy(bits.view(np.int16)).to(dev).view(torch.bfloat16)
+    a = torch.zeros(1, dtype=torch.float32, device=dev)
+    assert pkg.FMHAAbsMaxBF16(None, xd, bits.size, a) == pkg.FMHA_I8_OK
+    q, _ = pkg.quantize_tensor(xd, amax=127.0)
+    torch.cuda.synchronize()
+    assert a.item() == float("inf")
+    assert list(q.cpu().numpy()) == [0, 1, 0, -2, 0, 0, 1, 2, 127]
