@@ -193,16 +193,17 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // before the first operand read of the current one.  Completion is tracked by hand with s_waitcnt vmcnt(n) in front
   // of the barrier that publishes a tile.  M0 carries the LDS destination of lane 0; lane l lands 16*l bytes further.
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) int8_t*)&lds[0][0][0];
-  auto issue_tile = [&](const int8_t* gbase, int kb, int which, int goff) {  // which: 0 = K, 1 = V
+  auto issue_region = [&](const int8_t* gbase, int kb, int which, int goff, int it) {  // which: 0 = K, 1 = V
     const int8_t* gp = gbase + (long)kb * kTileBytes;  // wave-uniform base (SGPR pair)
     if (RAGGED && kb == tail_kb) gp = gbase + (long)(S - BK) * D;
+    const int region = (it * kWaves + wave) % kRegions;
+    const unsigned dst = lds_base + (unsigned)(((kb & (kStages - 1)) * 2 + which) * kTileBytes + region * 1024);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(dst), "v"(goff + region * 1024), "s"(gp) : "memory");
+  };
+  auto issue_tile = [&](const int8_t* gbase, int kb, int which, int goff) {
 #pragma unroll
-    for (int it = 0; it < kRegionsPerWave; ++it) {
-      const int region = (it * kWaves + wave) % kRegions;
-      const unsigned dst = lds_base + (unsigned)(((kb & (kStages - 1)) * 2 + which) * kTileBytes + region * 1024);
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                   :: "s"(dst), "v"(goff + region * 1024), "s"(gp) : "memory");
-    }
+    for (int it = 0; it < kRegionsPerWave; ++it) issue_region(gbase, kb, which, goff, it);
   };
   auto issue_k = [&](int kb) { issue_tile(kg, kb, 0, ld_goff_k); };
   auto issue_v = [&](int kb) { issue_tile(vg, kb, 1, ld_goff_v); };
@@ -494,7 +495,13 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // (inc/fmha_i8.cuh:298-315) four elements behind each MFMA of tile u.  Normalisation is deferred to the epilogue:
   // O and l are kept relative to 2^m_ref, and m_ref only moves when some row's block maximum exceeds it by
   // 2^kLazyLog2.
-  auto phase_gemm2_merge = [&](int kb, const v4i (&pk)[kKeyTiles]) {
+  // Where the tile loads of a block are issued: at the end of the softmax phase, or one per output tile inside GEMM 2.
+  // The loads and their address arithmetic stand in the issue stream of whichever wavefront carries them, and the
+  // barrier waits for the longer stream: at d = 64 that is the softmax wavefront (the MFMA phase is short: -7 % with
+  // the loads moved there), at d = 128 the two are level and the loads stay where the wavefront used to arrive early.
+  constexpr bool kLoadsInMfmaPhase = D == 64;
+  static_assert(!kLoadsInMfmaPhase || 2 * kRegionsPerWave <= kDSteps, "one tile load per output tile of GEMM 2");
+  auto phase_gemm2_merge = [&](int kb, const v4i (&pk)[kKeyTiles], int k_next, int v_next) {
     if (__ballot(m_blk > m_ref + kLazyLog2) != 0) {
       const float m_new = fmaxf(m_ref, m_blk);
       const float keep = __builtin_amdgcn_exp2f(m_ref - m_new);
@@ -545,6 +552,11 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
           __builtin_amdgcn_sched_barrier(0);
         }
       }
+      if (kLoadsInMfmaPhase) {
+        if (u < kRegionsPerWave) issue_region(kg, k_next, 0, ld_goff_k, u);
+        else if (u < 2 * kRegionsPerWave) issue_region(vg, v_next, 1, ld_goff_v, u - kRegionsPerWave);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) merge_piece(oacc[(kDSteps - 1) & 1], kDSteps - 1, j);
@@ -575,13 +587,16 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       issue_v(min(1, last));
     }
   };
-  auto issue_after_softmax = [&](int i) {
+  auto issue_for = [&](int i) {  // where GEMM 2 of block i is skipped
     issue_k(min(i + 3, last));
     issue_v(min(i + 2, last));
   };
-  // Before barrier 2m every wavefront waits for its share of K(m) and V(m-1).  Tiles issued later may stay in flight:
-  // K(m+1), V(m) (after Y(m-2)) and, for the wavefronts that have already finished Y(m-1), K(m+2), V(m+1).
-  auto wait_tiles_for = [&](bool after_next_softmax) { wait_all_but(after_next_softmax ? 4 : 2); };
+  // Before barrier 2m every wavefront waits for its share of K(m) and V(m-1).  The tiles issued since may stay in
+  // flight: the pair of the previous issue point and, for wavefronts 0..3 when they issue after the softmax (they
+  // have just done so), the pair of this one.
+  auto wait_tiles = [&](bool issued_after_softmax) { wait_all_but(!kLoadsInMfmaPhase && issued_after_softmax ? 4 : 2); };
+  auto issue_after_softmax = [&](int i) { if (!kLoadsInMfmaPhase) issue_for(i); };
+  auto issue_in_mfma_phase = [&](int i) { if (kLoadsInMfmaPhase) issue_for(i); };
   v16i acc[kKeyTiles];  // S^T of the block whose softmax comes next (GEMM 1 -> softmax, across a barrier)
   int mx[2];
   // Where GEMM 1 is skipped the old scores are dead; saying so (an empty definition) keeps 64 registers from being
@@ -610,10 +625,10 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         barrier();
         phase_softmax(i, 0, acc, pk, mx);
         issue_after_softmax(i);
-        wait_tiles_for(true);
+        wait_tiles(true);
         barrier();
         raise_priority();
-        phase_gemm2_merge(i, pk);
+        phase_gemm2_merge(i, pk, min(i + 3, last), min(i + 2, last));
         phase_gemm1(i + 1, acc, mx);
         drop_priority();
       }
@@ -625,10 +640,11 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       barrier();                               // barrier 2i+1
       if (work) phase_softmax(i, cls, acc, pk, mx);
       issue_after_softmax(i);
-      wait_tiles_for(true);
+      wait_tiles(true);
       barrier();                               // barrier 2i+2
       raise_priority();
-      if (work) phase_gemm2_merge(i, pk);
+      if (work) phase_gemm2_merge(i, pk, min(i + 3, last), min(i + 2, last));
+      else issue_in_mfma_phase(i);
       if (i + 1 < n && works(i + 1)) phase_gemm1(i + 1, acc, mx);
       else forget_scores();
       drop_priority();
@@ -643,13 +659,13 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     if (active) {  // steady state, see above
       for (; i + 1 < n && i + 1 < kb_plain; ++i) {
         v4i pk[kKeyTiles];
-        wait_tiles_for(false);
+        wait_tiles(false);
         barrier();
         phase_softmax(i, 0, acc, pk, mx);
         issue_after_softmax(i);
         barrier();
         raise_priority();
-        phase_gemm2_merge(i, pk);
+        phase_gemm2_merge(i, pk, min(i + 3, last), min(i + 2, last));
         phase_gemm1(i + 1, acc, mx);
         drop_priority();
       }
@@ -658,13 +674,14 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       const int cls = cls_of(i);
       const bool work = active && !(cls & 2);
       v4i pk[kKeyTiles];
-      wait_tiles_for(false);
+      wait_tiles(false);
       barrier();                               // barrier 2i+2
       if (work) phase_softmax(i, cls, acc, pk, mx);
       issue_after_softmax(i);
       barrier();                               // barrier 2i+3
       raise_priority();
-      if (work) phase_gemm2_merge(i, pk);
+      if (work) phase_gemm2_merge(i, pk, min(i + 3, last), min(i + 2, last));
+      else issue_in_mfma_phase(i);
       if (i + 1 < n && works(i + 1)) phase_gemm1(i + 1, acc, mx);
       else forget_scores();
       drop_priority();
