@@ -11,6 +11,9 @@ simulates:
   block_local  flash-style: per block of 128 keys (64 when the length is not a multiple of 128), p = exp(x - block
                maximum) quantised with scale 128, row sum kept un-quantised, blocks merged online
                (inc/fmha_i8.cuh:181-253,298-315)
+  block_local_full
+               the same with 255 steps: the "uint8 x int8" variant the reference plans (README.md:15,186), which on
+               int8 matrix hardware would be P - 128 as int8 plus 128 times the column sums of V per block
   kernel       (optional, --kernel) the HIP kernel itself through libfmha_i8.so, int8 output de-quantised with
                o_amax = max |float O|; adds the output quantisation on top of block_local; multiples of 64 only
 
@@ -34,7 +37,7 @@ import sys
 import numpy as np
 
 SOFTMAX_QUANT_SCALE = 127  # fmha_i8_quant_error_seqlen.py:4
-SCHEMES = ("worst", "static", "dynamic", "block_local")
+SCHEMES = ("worst", "static", "dynamic", "block_local", "block_local_full")
 f32 = np.float32
 
 
@@ -60,8 +63,9 @@ def block_keys_for(seq_len):
     return 128 if seq_len % 128 == 0 else 64  # src/fmha_i8.cu:39-154
 
 
-def block_local_attention(s_f, v_i8, v_amax, block):
-    """The kernel's scheme on de-quantised scores s_f [S, S_kv] (float32) and int8 V: returns float O [S, d]."""
+def block_local_attention(s_f, v_i8, v_amax, block, steps=128):
+    """The kernel's scheme on de-quantised scores s_f [S, S_kv] (float32) and int8 V: returns float O [S, d].
+    steps: quantisation steps of P (128 in the kernel: p = 1 maps to -128)."""
     S = s_f.shape[0]
     m_run = np.full(S, -np.inf, f32)
     l_run = np.zeros(S, f32)
@@ -71,14 +75,14 @@ def block_local_attention(s_f, v_i8, v_amax, block):
         m_blk = x.max(axis=1)
         p = np.exp(x - m_blk[:, None]).astype(f32)
         l_blk = p.sum(axis=1, dtype=f32)                                   # un-quantised (inc/fmha_i8.cuh:208-235)
-        p_q = np.rint(np.clip(f32(128.0) * p, 0, 128)).astype(np.int32)    # |P| of inc/fmha_i8.cuh:241,249
+        p_q = np.rint(np.clip(f32(steps) * p, 0, steps)).astype(np.int32)  # |P| of inc/fmha_i8.cuh:241,249
         o_blk = (p_q @ v_i8[k0:k0 + block].astype(np.int32)).astype(f32)   # exact int32
         m_new = np.maximum(m_run, m_blk)
         a, b = np.exp(m_run - m_new).astype(f32), np.exp(m_blk - m_new).astype(f32)
         l_run = a * l_run + b * l_blk
         o_run = a[:, None] * o_run + b[:, None] * o_blk
         m_run = m_new
-    return (o_run / (f32(128.0) * l_run)[:, None]) * f32(v_amax / 127.0)
+    return (o_run / (f32(steps) * l_run)[:, None]) * f32(v_amax / 127.0)
 
 
 def simulate(seq_len, head_dim, rng, kernel=None, levels=SOFTMAX_QUANT_SCALE):
@@ -101,6 +105,7 @@ def simulate(seq_len, head_dim, rng, kernel=None, levels=SOFTMAX_QUANT_SCALE):
     out["static"] = through_uint8(float(np.abs(f_p).max()))
     out["dynamic"] = through_uint8(p.max(axis=1, keepdims=True))
     out["block_local"] = block_local_attention(s_f.astype(f32), i8_v, v_amax, block_keys_for(seq_len))
+    out["block_local_full"] = block_local_attention(s_f.astype(f32), i8_v, v_amax, block_keys_for(seq_len), steps=255)
     o_amax = float(np.abs(out["ref"]).max())
     out.update(q=i8_q, k=i8_k, v=i8_v, q_amax=q_amax, k_amax=k_amax, v_amax=v_amax, o_amax=o_amax)
     if kernel is not None and seq_len % 64 == 0:
