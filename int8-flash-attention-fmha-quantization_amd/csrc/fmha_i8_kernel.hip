@@ -564,14 +564,16 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 
   // ---- the tick schedule -------------------------------------------------------------------------------------------
   // A tick is the interval between two workgroup barriers.  Every key block i is two phases per wavefront: an MFMA
-  // phase M(i) = [GEMM 2 + merge of block i-1][GEMM 1 of block i], bound by LDS operand reads, and a VALU phase
-  // Y(i) = softmax of block i.  Wavefronts 0..3 run M(i) in tick 2i and Y(i) in tick 2i+1; wavefronts 4..7 run one tick
-  // behind, so the MFMA phase of one always overlaps the VALU phase of the other wavefront of the same SIMD.
+  // phase M(i) = [GEMM 2 + merge of block i-1][GEMM 1 of block i] and a VALU phase Y(i) = softmax of block i.
+  // Wavefronts 0..3 run M(i) in tick 2i and Y(i) in tick 2i+1; wavefronts 4..7 run one tick behind, so the MFMA phase
+  // of one always overlaps the VALU phase of the other wavefront of the same SIMD.  The two share one issue port: a
+  // tick lasts about as long as the issue time of both phases together, and the barrier waits for the wavefront whose
+  // own instruction stream - vector, scalar and memory instructions alike - is the longer one.
   // Tiles: K(j), V(j) live in stage j mod 4; K(j) is read in ticks 2j and 2j+1, V(j) in ticks 2j+2 and 2j+3, and
   // barrier 2m publishes K(m) and V(m-1).  A wavefront is held for hundreds of cycles when it issues loads (the CU's
-  // vector memory path takes 64 bytes per cycle and all eight wavefronts queue up), so it issues at the END of its
-  // softmax phase, the one place where it would otherwise reach the barrier early: K(i+3) and V(i+2) after Y(i).  Both
-  // stages were last read in tick 2i-1.  Issue order per wavefront: K0 V0 | K1 K2 V1 | K3 V2 | K4 V3 | ...
+  // vector memory path takes 64 bytes per cycle and all eight wavefronts queue up).  K(i+3) and V(i+2) are issued
+  // after Y(i), at the end of the softmax phase, or (d = 64) inside the MFMA phase that follows it; both stages were
+  // last read in tick 2i-1.  Issue order per wavefront: K0 V0 | K1 K2 V1 | K3 V2 | K4 V3 | ...
   const int n = kb_end;
   auto cls_of = [&](int kb) { return __builtin_amdgcn_readfirstlane((int)lds_class[kb]); };
   auto works = [&](int kb) { return active && !(cls_of(kb) & 2); };  // nothing in a fully masked block is attended to
