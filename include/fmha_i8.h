@@ -20,8 +20,9 @@
  * 192, 256, 320, 384, 448, 512, 1024, 2048, 4096.  All of them are covered here, and so is every other length.
  * As in the reference, the softmax works on blocks of 128 keys when seq_len is a multiple of 128 and on blocks of 64 keys
  * when it is another multiple of 64 - the block size is part of the numerics, because P is quantised against the
- * BLOCK-LOCAL row maximum.  A length that is not a multiple of 64 gives exactly what the caller would get by padding
- * K, V and the mask to the next multiple of 64 with masked keys; the library does it without the copies.)
+ * BLOCK-LOCAL row maximum.  A length that is not a multiple of 64 gives what the caller would get by padding K, V and
+ * the mask to the next multiple of 64 with masked keys (the float row sum of the last block adds its terms in another
+ * order, nothing else differs); the library does it without the copies and never reads past the last key.)
  *
  * Numerics follow the reference kernel (inc/fmha_i8.cuh:71-72,181-253,298-332): int32 Q.K^T, 1/sqrt(d) and
  * q_amax*k_amax/127^2 dequantisation, softmax over blocks of 128 (or 64) keys with the BLOCK-LOCAL row maximum,
