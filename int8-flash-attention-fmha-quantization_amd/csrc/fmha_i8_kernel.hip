@@ -193,7 +193,23 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // before the first operand read of the current one.  Completion is tracked by hand with s_waitcnt vmcnt(n) in front
   // of the barrier that publishes a tile.  M0 carries the LDS destination of lane 0; lane l lands 16*l bytes further.
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) int8_t*)&lds[0][0][0];
+  // Tile 0 of a sequence shorter than one block - the only tile there is, fetched in the prologue and again at every
+  // later issue point: rows past the last key fetch the last key instead (same chunk: the swizzle belongs to the LDS
+  // row); what lands there is never attended to, those keys are masked.  Fetching the whole tile would read up to
+  // BK - S rows past the end of K and V.
+  auto issue_short_region = [&](const int8_t* gbase, int which, int goff, int it) {
+    const int region = (it * kWaves + wave) % kRegions;
+    const unsigned dst = lds_base + (unsigned)(which * kTileBytes + region * 1024);
+    const int row = region * kRowsPerRegion + ld_row_in;
+    const int src = goff + region * 1024 - (row >= S ? (row - (S - 1)) * D : 0);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(dst), "v"(src), "s"(gbase) : "memory");
+  };
   auto issue_region = [&](const int8_t* gbase, int kb, int which, int goff, int it) {  // which: 0 = K, 1 = V
+    if (RAGGED && short_seq) {
+      issue_short_region(gbase, which, goff, it);
+      return;
+    }
     const int8_t* gp = gbase + (long)kb * kTileBytes;  // wave-uniform base (SGPR pair)
     if (RAGGED && kb == tail_kb) gp = gbase + (long)(S - BK) * D;
     const int region = (it * kWaves + wave) % kRegions;
@@ -207,19 +223,6 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   };
   auto issue_k = [&](int kb) { issue_tile(kg, kb, 0, ld_goff_k); };
   auto issue_v = [&](int kb) { issue_tile(vg, kb, 1, ld_goff_v); };
-  // tile 0 of a sequence shorter than one block (prologue only): rows past the last key fetch the last key instead
-  // (same chunk: the swizzle belongs to the LDS row); what lands there is never attended to, those keys are masked
-  auto issue_short = [&](const int8_t* gbase, int which, int goff) {
-#pragma unroll
-    for (int it = 0; it < kRegionsPerWave; ++it) {
-      const int region = (it * kWaves + wave) % kRegions;
-      const unsigned dst = lds_base + (unsigned)(which * kTileBytes + region * 1024);
-      const int row = region * kRowsPerRegion + ld_row_in;
-      const int src = goff + region * 1024 - (row >= S ? (row - (S - 1)) * D : 0);
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                   :: "s"(dst), "v"(src), "s"(gbase) : "memory");
-    }
-  };
   // Memory reads return in issue order: waiting until at most `tiles` tiles of this wavefront's loads are outstanding
   // retires every tile older than the newest `tiles` ones.
   auto wait_all_but = [&](int tiles) {
@@ -244,8 +247,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     const int j = 4 * tid + 4 <= S ? 4 * tid : S - 4;
     asm volatile("global_load_dword %0, %1, %2" : "=v"(mask_word) : "v"(j), "s"(mg) : "memory");
   }
-  if (short_seq) issue_short(kg, 0, ld_goff_k);
-  else issue_k(0);
+  issue_k(0);
   v4i qreg[kDSteps];  // Q: B operand of GEMM 1, loaded once
   {
     // rows past the end of the sequence load the last row (unused) so that every wavefront has the same loads in flight
@@ -256,8 +258,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     for (int kk = 0; kk < kDSteps; ++kk)
       asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(qreg[kk]) : "v"(qoff + 32 * kk), "s"(qp) : "memory");
   }
-  if (short_seq) issue_short(vg, 1, ld_goff_v);
-  else issue_v(0);
+  issue_v(0);
 
   // ---- classify the key blocks of this batch entry: 4 mask bytes per lane, BK/4 lanes per block ---------------------
   asm volatile("s_waitcnt vmcnt(%1)" : "+v"(mask_word) : "n"(2 * kRegionsPerWave + kDSteps) : "memory");

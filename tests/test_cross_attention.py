@@ -209,3 +209,54 @@ def test_any_key_count_at_the_end_of_an_allocation(pkg, orc, dev):
     o = pkg.fmha_infer_i8(qd, bufs[0][1], bufs[1][1], bufs[2][1], *_scales(c))
     torch.cuda.synchronize()
     _gate(o.cpu().numpy(), want, "end of allocation")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("S,d", [(3, 64), (19, 128), (58, 64), (100, 128)])
+def test_sequences_shorter_than_one_block_with_many_query_blocks(pkg, orc, dev, S, d):
+    """A key sequence shorter than one block has a single tile, which every later issue point of the key loop fetches
+    again: each of those fetches has to stop at the last key like the first one does (tiny K and V tensors, several
+    heads and query blocks, so that a full-tile fetch would run far past their end)."""
+    B, H, Sq = 3, 3, 319
+    c = fc.make_inputs(B, H, 128, d, seed=64)
+    k, v = (np.ascontiguousarray(c[n][:, :, :S]) for n in ("k", "v"))
+    mask = np.zeros((B, S), np.int8)
+    mask[1, S // 2 + 1:] = 1
+    q = fc.make_inputs(B, H, Sq, d, seed=65)["q"]
+    cc = dict(c, k=k, v=v, mask=mask)
+    _gate(_gpu(pkg, dev, q, cc, canary=True), orc.fmha_i8_blockwise_cross(q, k, v, mask, *_scales(c)),
+          "short S=%d d=%d" % (S, d))
+
+
+@pytest.mark.gpu
+def test_random_shapes(pkg, orc, dev):
+    """Sixty seeded random problems - any query count, any key count, every kind of mask (none, scattered, ragged
+    tails, a run of fully masked blocks in the middle), both head sizes, both distributions, three score scales -
+    against the checker with the usual gate."""
+    import torch
+    rng = np.random.default_rng(2024)
+    for it in range(60):
+        d = int(rng.choice([64, 128]))
+        B, H = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        S = int(rng.choice([rng.integers(1, 130), rng.integers(1, 700), rng.integers(500, 2600), 64 * rng.integers(1, 40)]))
+        Sq = S if rng.random() < 0.4 else int(rng.choice([rng.integers(1, 70), rng.integers(1, 600), rng.integers(200, 1500)]))
+        pad = str(rng.choice(["none", "scatter", "tail", "dead"]))
+        c = fc.make_inputs(B, H, (S + 63) // 64 * 64, d, pad="scatter" if pad == "scatter" else "none", seed=1000 + it,
+                           dist=str(rng.choice(["normal", "student_t"])), sigma=float(rng.choice([0.5, 1.0])))
+        mask = c["mask"][:, :S].copy()
+        if pad == "tail":
+            for b in range(B):
+                mask[b, int(rng.integers(1, S + 1)):] = 1
+        if pad == "dead" and S > 256:
+            a = int(rng.integers(0, S - 130))
+            mask[:, a:a + int(rng.integers(64, 400))] = 1
+        mask[:, 0] = 0
+        k, v = (np.ascontiguousarray(c[n][:, :, :S]) for n in ("k", "v"))
+        q = fc.make_inputs(B, H, Sq, d, seed=5000 + it)["q"]
+        scales = (c["q_amax"] * float(rng.choice([1, 1, 8, 40])), c["k_amax"], c["v_amax"], float(rng.choice([1.0, 2.0])))
+        print("case", it, B, H, Sq, S, d, pad, flush=True)
+        want = orc.fmha_i8_blockwise_cross(q, k, v, mask, *scales)
+        t = [torch.from_numpy(np.ascontiguousarray(a)).to(dev) for a in (q, k, v, mask)]
+        got = pkg.fmha_infer_i8(*t, *scales)
+        torch.cuda.synchronize()
+        _gate(got.cpu().numpy(), want, "random case %d" % it)
