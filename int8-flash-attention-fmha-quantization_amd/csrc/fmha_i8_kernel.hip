@@ -203,7 +203,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     const int row = region * kRowsPerRegion + ld_row_in;
     const int src = goff + region * 1024 - (row >= S ? (row - (S - 1)) * D : 0);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(dst), "v"(src), "s"(gbase) : "memory");
+                 :: "s"(dst), "v"(src), "s"(gbase) : "memory", "m0");
   };
   auto issue_region = [&](const int8_t* gbase, int kb, int which, int goff, int it) {  // which: 0 = K, 1 = V
     if (RAGGED && short_seq) {
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     const int region = (it * kWaves + wave) % kRegions;
     const unsigned dst = lds_base + (unsigned)(((kb & (kStages - 1)) * 2 + which) * kTileBytes + region * 1024);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(dst), "v"(goff + region * 1024), "s"(gp) : "memory");
+                 :: "s"(dst), "v"(goff + region * 1024), "s"(gp) : "memory", "m0");
   };
   auto issue_tile = [&](const int8_t* gbase, int kb, int which, int goff) {
 #pragma unroll
