@@ -150,6 +150,18 @@ const char* FMHAInferI8StatusString(int status) {
   return "unknown status";
 }
 
+#ifdef FMHA_CHECK_BOUNDS
+// Test build only: the number of global accesses that would have left their tensor since the last call of this
+// function (synchronises the device; see the kernel source).
+int FMHAInferI8DebugOutOfBounds(void) {
+  int count = -1, zero = 0;
+  if (hipDeviceSynchronize() != hipSuccess) return -1;
+  if (hipMemcpyFromSymbol(&count, HIP_SYMBOL(fmha_i8_gfx950::g_fmha_oob_count), sizeof(int)) != hipSuccess) return -1;
+  if (hipMemcpyToSymbol(HIP_SYMBOL(fmha_i8_gfx950::g_fmha_oob_count), &zero, sizeof(int)) != hipSuccess) return -1;
+  return count;
+}
+#endif
+
 const char* FMHAInferI8Version(void) { return "fmha_i8 gfx950 mfma32x32x32 direct-to-lds two-phase"; }
 
 }  // extern "C"

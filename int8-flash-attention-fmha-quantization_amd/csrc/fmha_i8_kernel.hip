@@ -56,6 +56,20 @@ constexpr float kBiasOffsetLimit = 4096.0f;  // see the launch code: bound on th
 constexpr float kLog2Pscale = -7.99995597f;  // log2(128 / 32767): exp2(x + kLog2Pscale) = 128 p / 32767
 constexpr float kLazyLog2 = 10.0f;       // the running O is rescaled only when a row maximum grows by more than this
 
+// FMHA_CHECK_BOUNDS (a test build, never the shipped library): every global access of the kernel is first checked
+// against the tensor - for K and V the head - it belongs to; an access that would leave it is counted in
+// g_fmha_oob_count and redirected to the first byte, so that the run ends normally and the test can read the count.
+// An out-of-bounds READ changes no result and, inside a caching allocator's pool, raises no fault: nothing else shows it.
+#ifdef FMHA_CHECK_BOUNDS
+__device__ int g_fmha_oob_count;
+__device__ __forceinline__ bool fmha_in_bounds(bool ok) {
+  if (!ok) atomicAdd(&g_fmha_oob_count, 1);
+  return ok;
+}
+#else
+__device__ __forceinline__ constexpr bool fmha_in_bounds(bool) { return true; }
+#endif
+
 struct KernelArgs {
   const int8_t* q;
   const int8_t* k;
@@ -201,9 +215,10 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     const int region = (it * kWaves + wave) % kRegions;
     const unsigned dst = lds_base + (unsigned)(which * kTileBytes + region * 1024);
     const int row = region * kRowsPerRegion + ld_row_in;
-    const int src = goff + region * 1024 - (row >= S ? (row - (S - 1)) * D : 0);
+    int src = goff + region * 1024 - (row >= S ? (row - (S - 1)) * D : 0);
+    if (!fmha_in_bounds(src >= 0 && src + 16 <= S * D)) src = 0;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(dst), "v"(src), "s"(gbase) : "memory", "m0");
+                 :: "s"(dst), "v"(src), "s"(gbase) : "memory");
   };
   auto issue_region = [&](const int8_t* gbase, int kb, int which, int goff, int it) {  // which: 0 = K, 1 = V
     if (RAGGED && short_seq) {
@@ -214,8 +229,13 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     if (RAGGED && kb == tail_kb) gp = gbase + (long)(S - BK) * D;
     const int region = (it * kWaves + wave) % kRegions;
     const unsigned dst = lds_base + (unsigned)(((kb & (kStages - 1)) * 2 + which) * kTileBytes + region * 1024);
+    int src = goff + region * 1024;
+    {
+      const long rel = (long)(gp - gbase) + src;  // offset inside the head
+      if (!fmha_in_bounds(rel >= 0 && rel + 16 <= (long)S * D)) src = (int)(gbase - gp);
+    }
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(dst), "v"(goff + region * 1024), "s"(gp) : "memory", "m0");
+                 :: "s"(dst), "v"(src), "s"(gp) : "memory");
   };
   auto issue_tile = [&](const int8_t* gbase, int kb, int which, int goff) {
 #pragma unroll
@@ -244,7 +264,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   const bool active = row0 < Sq;              // the last workgroup of a head may be partly empty
   int mask_word = 0;
   if (!RAGGED || S >= 4) {  // (a shorter mask row has no dword that lies inside it)
-    const int j = 4 * tid + 4 <= S ? 4 * tid : S - 4;
+    int j = 4 * tid + 4 <= S ? 4 * tid : S - 4;
+    if (!fmha_in_bounds(j >= 0 && j + 4 <= S)) j = 0;
     asm volatile("global_load_dword %0, %1, %2" : "=v"(mask_word) : "v"(j), "s"(mg) : "memory");
   }
   issue_k(0);
@@ -252,7 +273,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   {
     // rows past the end of the sequence load the last row (unused) so that every wavefront has the same loads in flight
     const int8_t* qp = args.q + q_head_off;
-    const int qrow = row0 + i32 < Sq ? row0 + i32 : Sq - 1;
+    int qrow = row0 + i32 < Sq ? row0 + i32 : Sq - 1;
+    if (!fmha_in_bounds(qrow >= 0 && qrow < Sq)) qrow = 0;
     const int qoff = qrow * D + 16 * g;
 #pragma unroll
     for (int kk = 0; kk < kDSteps; ++kk)
@@ -270,10 +292,11 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         const unsigned w = (unsigned)mask_word;
         nib = ((w & 0xffu) ? 1 : 0) | ((w & 0xff00u) ? 2 : 0) | ((w & 0xff0000u) ? 4 : 0) | ((w & 0xff000000u) ? 8 : 0);
       } else {
-        nib = (mg[j] != 0 ? 1 : 0) | (mg[j + 1] != 0 ? 2 : 0) | (mg[j + 2] != 0 ? 4 : 0) | (mg[j + 3] != 0 ? 8 : 0);
+        const int jj = fmha_in_bounds(j >= 0 && j + 4 <= S) ? j : 0;
+        nib = (mg[jj] != 0 ? 1 : 0) | (mg[jj + 1] != 0 ? 2 : 0) | (mg[jj + 2] != 0 ? 4 : 0) | (mg[jj + 3] != 0 ? 8 : 0);
       }
     } else if (RAGGED && j < S) {  // the one lane that straddles the end
-      for (int b = 0; b < S - j; ++b) nib = (mg[j + b] != 0) ? nib : (nib & ~(1 << b));
+      for (int b = 0; b < S - j; ++b) nib = (mg[fmha_in_bounds(j + b < S) ? j + b : 0] != 0) ? nib : (nib & ~(1 << b));
     }
     // eight lanes hold the 32 mask bits of one word
     unsigned word = (unsigned)nib << (4 * (lane & 7));
@@ -714,6 +737,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // both words of output tile u and lane l+32 both words of tile u+1: every lane then owns 32 contiguous bytes of a
   // row and writes them with two 128-bit stores instead of eight scattered 32-bit ones.
   if (row0 + i32 >= Sq) return;  // (no barrier follows)
+  if (!fmha_in_bounds(row0 + i32 >= 0 && q_head_off + (long)(row0 + i32 + 1) * D <= (long)args.total_wgs / args.q_blocks * Sq * D))
+    return;
   int8_t* op = args.o + q_head_off + (long)(row0 + i32) * D + 32 * g;
 #pragma unroll
   for (int u = 0; u < kDSteps; u += 2) {
