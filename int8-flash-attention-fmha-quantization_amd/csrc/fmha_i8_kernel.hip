@@ -461,6 +461,11 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       // off = top*c2 rounded; p' = exp2(s*c2 - off) = p * 2^(resid) with one row-wide resid below 1 ulp of off, and the
       // block maximum that is consistent with p' is off itself (minus the constant kBase*c2 when BIAS).
       float off = top * c2;
+      // Where the scores are converted, c2 is large and |off| can reach 10^5 and more: the rounding of this product and
+      // of offq below then amounts to a percent of p, and a p above 1 by 0.4 % quantises to -129, whose low byte is
+      // +127.  Two units in the last place upwards make off an upper bound of the exact product: every p is at most 1,
+      // the row is scaled by one common factor just below 1 (l with it: the output does not notice).
+      if (!BIAS) off = __builtin_fmaf(fabsf(off), 2.384185791015625e-07f, off);
       if (!BIAS) off = fmaxf(off, args.floor2);
       m_blk = off - bias_c2;
       const float offq = off - kLog2Pscale;  // exp2(x - offq) = 128 p / 32767: the snorm conversion returns rne(128 p)

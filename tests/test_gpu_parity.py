@@ -286,6 +286,21 @@ def test_negative_score_scale_is_refused(pkg, dev):
     assert (o == 55).all().item()
 
 
+def test_exponent_offsets_of_the_order_of_a_hundred_thousand(pkg, orc, dev):
+    """Heavy-tailed Q, K and a forty-fold score scale: block maxima of 10^5 in base-2 units, where one unit in the last
+    place of the offset is a percent of p.  The largest p of a row must still quantise to at most 128 in magnitude (it
+    once reached 129, whose low byte is +127: two rows of this very problem came out with the wrong sign)."""
+    import torch
+    c = fc.make_inputs(2, 3, 1152, 64, dist="student_t", sigma=1.0, seed=1128)
+    q = fc.make_inputs(2, 3, 470, 64, seed=5128)["q"]
+    scales = (c["q_amax"] * 40.0, c["k_amax"], c["v_amax"], 1.0)
+    want = orc.fmha_i8_blockwise_cross(q, c["k"], c["v"], c["mask"], *scales)
+    t = to_dev(dev, q, c["k"], c["v"], c["mask"])
+    got = pkg.fmha_infer_i8(*t, *scales)
+    torch.cuda.synchronize()
+    check(got.cpu().numpy(), want, "large offsets")
+
+
 def test_masked_sentinel_corner(pkg, orc, dev):
     # every unmasked score of a partially masked block lies below the -1,000,000 substituted for masked keys
     S, d = 128, 128
