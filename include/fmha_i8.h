@@ -87,6 +87,15 @@ typedef struct FMHACrossAttnDescriptor {
 int FMHAInferI8Cross(hipStream_t stream, FMHAParamI8 fmha_param, FMHACrossAttnDescriptor desc, const void* q,
                      const void* k, const void* v, const void* padding_mask, void* o);
 
+/* FMHAInferI8Cross with P on all 255 steps of a byte: P = rne(255 p) in [0, 255] where the reference's kernel has
+ * rne(-128 p) in [-128, 0] (inc/fmha_i8.cuh:241,249) - the "uint8 x int8" variant that the reference lists as planned
+ * and has no code for (README.md:15,186).  Same arguments, layouts, scales, status codes and asynchrony; the output
+ * differs from FMHAInferI8Cross's by at most a few LSBs and is closer to the unquantised attention (P carries one bit
+ * more).  About a tenth slower: the matrix unit multiplies signed bytes only, so the kernel computes with P - 128 and
+ * adds 128 times the column sums of every V tile. */
+int FMHAInferI8CrossFullRangeP(hipStream_t stream, FMHAParamI8 fmha_param, FMHACrossAttnDescriptor desc, const void* q,
+                               const void* k, const void* v, const void* padding_mask, void* o);
+
 /* Argument check only, no HIP call: what FMHAInferI8Cross would return before launching. */
 int FMHAInferI8CrossCheckArgs(FMHAParamI8 fmha_param, FMHACrossAttnDescriptor desc, const void* q, const void* k,
                               const void* v, const void* padding_mask, const void* o);

@@ -16,8 +16,9 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libfmha_i8.so")
 
 EXPORTED_SYMBOLS = ("FMHAInferI8", "FMHAInferI8Status", "FMHAInferI8CheckArgs", "FMHAInferI8StatusString",
-                    "FMHAInferI8Version", "FMHAInferI8Cross", "FMHAInferI8CrossCheckArgs", "FMHAAbsMaxF32",
-                    "FMHAQuantizeI8", "FMHADequantizeI8", "FMHAAbsMaxBF16", "FMHAQuantizeI8BF16", "FMHADequantizeI8BF16")
+                    "FMHAInferI8Version", "FMHAInferI8Cross", "FMHAInferI8CrossCheckArgs",
+                    "FMHAInferI8CrossFullRangeP", "FMHAAbsMaxF32", "FMHAQuantizeI8", "FMHADequantizeI8",
+                    "FMHAAbsMaxBF16", "FMHAQuantizeI8BF16", "FMHADequantizeI8BF16")
 
 FMHA_I8_OK = 0
 FMHA_I8_ERR_NULL_POINTER = 1
@@ -92,6 +93,8 @@ def load_library(path=None):
     L.FMHAInferI8Version.restype = C.c_char_p
     L.FMHAInferI8Cross.argtypes = [ptr, FMHAParamI8, FMHACrossAttnDescriptor, ptr, ptr, ptr, ptr, ptr]
     L.FMHAInferI8Cross.restype = C.c_int
+    L.FMHAInferI8CrossFullRangeP.argtypes = L.FMHAInferI8Cross.argtypes
+    L.FMHAInferI8CrossFullRangeP.restype = C.c_int
     L.FMHAInferI8CrossCheckArgs.argtypes = [FMHAParamI8, FMHACrossAttnDescriptor, ptr, ptr, ptr, ptr, ptr]
     L.FMHAInferI8CrossCheckArgs.restype = C.c_int
     # include/fmha_quant.h
@@ -149,6 +152,12 @@ def FMHAInferI8Cross(stream, fmha_param, desc, q, k, v, padding_mask, o):
     """seq_len_q queries over seq_len_kv keys; status code of include/fmha_i8.h."""
     return int(load_library().FMHAInferI8Cross(_stream(stream), fmha_param, desc, _ptr(q), _ptr(k), _ptr(v),
                                                _ptr(padding_mask), _ptr(o)))
+
+
+def FMHAInferI8CrossFullRangeP(stream, fmha_param, desc, q, k, v, padding_mask, o):
+    """FMHAInferI8Cross with P = rne(255 p) on all 255 steps of a byte (README.md:15,186 of the reference plans it)."""
+    return int(load_library().FMHAInferI8CrossFullRangeP(_stream(stream), fmha_param, desc, _ptr(q), _ptr(k), _ptr(v),
+                                                         _ptr(padding_mask), _ptr(o)))
 
 
 def FMHAInferI8CrossCheckArgs(fmha_param, desc, q, k, v, padding_mask, o):
@@ -232,12 +241,14 @@ def dequantize_tensor(x, amax, stream=None, dtype=None):
     return out
 
 
-def fmha_infer_i8(q, k, v, padding_mask, q_amax, k_amax, v_amax, o_amax=1.0, out=None, stream=None):
+def fmha_infer_i8(q, k, v, padding_mask, q_amax, k_amax, v_amax, o_amax=1.0, out=None, stream=None,
+                  full_range_p=False):
     """Convenience over FMHAInferI8Status for torch int8 tensors on the GPU.
 
     q: int8 [B, H, Sq, d]; k, v: int8 [B, H, S, d], all contiguous; padding_mask: int8 [B, S], nonzero = key masked
     out (inc/fmha_i8.cuh:189-192).  Returns int8 O [B, H, Sq, d].  Sq == S goes through the reference's entry point
-    (FMHAInferI8Status), anything else through FMHAInferI8Cross.  Raises FMHAError on a nonzero status."""
+    (FMHAInferI8Status), anything else through FMHAInferI8Cross; full_range_p=True selects
+    FMHAInferI8CrossFullRangeP (P on 255 steps instead of 128).  Raises FMHAError on a nonzero status."""
     import torch
 
     for name, t in (("q", q), ("k", k), ("v", v), ("padding_mask", padding_mask)):
@@ -254,7 +265,10 @@ def fmha_infer_i8(q, k, v, padding_mask, q_amax, k_amax, v_amax, o_amax=1.0, out
     if stream is None:
         stream = torch.cuda.current_stream(q.device)
     param = FMHAParamI8(q_amax, k_amax, v_amax, o_amax, 1.0)
-    if Sq == S:
+    if full_range_p:
+        st = FMHAInferI8CrossFullRangeP(stream, param, FMHACrossAttnDescriptor(B, Sq, S, H, d), q, k, v, padding_mask,
+                                        out)
+    elif Sq == S:
         st = FMHAInferI8Status(stream, param, AttnDataDescriptor(B, S, H, d), q, k, v, padding_mask, out, True)
     else:
         st = FMHAInferI8Cross(stream, param, FMHACrossAttnDescriptor(B, Sq, S, H, d), q, k, v, padding_mask, out)

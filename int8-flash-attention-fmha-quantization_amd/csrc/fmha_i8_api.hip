@@ -36,22 +36,30 @@ int check_args(const FMHAParamI8& p, const FMHACrossAttnDescriptor& a, const voi
   return FMHA_I8_OK;
 }
 
-template <int D, int BK, bool RAGGED>
-void launch_variant3(bool bias, bool fast, dim3 grid, dim3 block, hipStream_t stream, const fmha_i8_gfx950::KernelArgs& args) {
+struct Variant {
+  bool bias, fast, full_range_p;
+};
+template <int D, int BK, bool RAGGED, bool FULLP>
+void launch_variant4(Variant var, dim3 grid, dim3 block, hipStream_t stream, const fmha_i8_gfx950::KernelArgs& args) {
   using namespace fmha_i8_gfx950;
-#define FMHA_LAUNCH(BB, FF) hipLaunchKernelGGL((fmha_i8_fwd_kernel<D, BK, BB, FF, RAGGED>), grid, block, 0, stream, args)
-  if (bias) { if (fast) FMHA_LAUNCH(true, true); else FMHA_LAUNCH(true, false); }
-  else { if (fast) FMHA_LAUNCH(false, true); else FMHA_LAUNCH(false, false); }
+#define FMHA_LAUNCH(BB, FF) hipLaunchKernelGGL((fmha_i8_fwd_kernel<D, BK, BB, FF, RAGGED, FULLP>), grid, block, 0, stream, args)
+  if (var.bias) { if (var.fast) FMHA_LAUNCH(true, true); else FMHA_LAUNCH(true, false); }
+  else { if (var.fast) FMHA_LAUNCH(false, true); else FMHA_LAUNCH(false, false); }
 #undef FMHA_LAUNCH
 }
+template <int D, int BK, bool RAGGED>
+void launch_variant3(Variant var, dim3 grid, dim3 block, hipStream_t stream, const fmha_i8_gfx950::KernelArgs& args) {
+  if (var.full_range_p) launch_variant4<D, BK, RAGGED, true>(var, grid, block, stream, args);
+  else launch_variant4<D, BK, RAGGED, false>(var, grid, block, stream, args);
+}
 template <int D, int BK>
-void launch_variant(bool bias, bool fast, dim3 grid, dim3 block, hipStream_t stream, const fmha_i8_gfx950::KernelArgs& args) {
-  if (args.seq_kv % BK != 0) launch_variant3<D, BK, true>(bias, fast, grid, block, stream, args);
-  else launch_variant3<D, BK, false>(bias, fast, grid, block, stream, args);
+void launch_variant(Variant var, dim3 grid, dim3 block, hipStream_t stream, const fmha_i8_gfx950::KernelArgs& args) {
+  if (args.seq_kv % BK != 0) launch_variant3<D, BK, true>(var, grid, block, stream, args);
+  else launch_variant3<D, BK, false>(var, grid, block, stream, args);
 }
 
 int launch(hipStream_t stream, const FMHAParamI8& p, const FMHACrossAttnDescriptor& a, const void* q, const void* k,
-           const void* v, const void* mask, void* o) {
+           const void* v, const void* mask, void* o, bool full_range_p = false) {
   const int st = check_args(p, a, q, k, v, mask, o);
   if (st != FMHA_I8_OK) return st;
   constexpr float kLog2e = 1.4426950408889634f;
@@ -91,12 +99,13 @@ int launch(hipStream_t stream, const FMHAParamI8& p, const FMHACrossAttnDescript
   const int block_keys = kv_padded % fmha_i8_gfx950::kBlockK == 0 ? fmha_i8_gfx950::kBlockK : fmha_i8_gfx950::kBlockKSmall;
   const float lsb_bound = 0.0034f * fabsf(p.v_amax / p.o_amax) * sqrtf((float)(kv_padded / block_keys));
   const bool fast = lsb_bound < 0.1f;
+  const Variant var{bias, fast, full_range_p};
   if (a.head_dim == 128) {
-    if (block_keys == fmha_i8_gfx950::kBlockK) launch_variant<128, fmha_i8_gfx950::kBlockK>(bias, fast, grid, block, stream, args);
-    else launch_variant<128, fmha_i8_gfx950::kBlockKSmall>(bias, fast, grid, block, stream, args);
+    if (block_keys == fmha_i8_gfx950::kBlockK) launch_variant<128, fmha_i8_gfx950::kBlockK>(var, grid, block, stream, args);
+    else launch_variant<128, fmha_i8_gfx950::kBlockKSmall>(var, grid, block, stream, args);
   } else {
-    if (block_keys == fmha_i8_gfx950::kBlockK) launch_variant<64, fmha_i8_gfx950::kBlockK>(bias, fast, grid, block, stream, args);
-    else launch_variant<64, fmha_i8_gfx950::kBlockKSmall>(bias, fast, grid, block, stream, args);
+    if (block_keys == fmha_i8_gfx950::kBlockK) launch_variant<64, fmha_i8_gfx950::kBlockK>(var, grid, block, stream, args);
+    else launch_variant<64, fmha_i8_gfx950::kBlockKSmall>(var, grid, block, stream, args);
   }
   const hipError_t err = hipGetLastError();
   return err == hipSuccess ? FMHA_I8_OK : FMHA_I8_ERR_HIP_BASE + (int)err;
@@ -119,6 +128,11 @@ int FMHAInferI8Status(hipStream_t stream, FMHAParamI8 fmha_param, AttnDataDescri
 int FMHAInferI8Cross(hipStream_t stream, FMHAParamI8 fmha_param, FMHACrossAttnDescriptor desc, const void* q,
                      const void* k, const void* v, const void* padding_mask, void* o) {
   return launch(stream, fmha_param, desc, q, k, v, padding_mask, o);
+}
+
+int FMHAInferI8CrossFullRangeP(hipStream_t stream, FMHAParamI8 fmha_param, FMHACrossAttnDescriptor desc, const void* q,
+                               const void* k, const void* v, const void* padding_mask, void* o) {
+  return launch(stream, fmha_param, desc, q, k, v, padding_mask, o, true);
 }
 
 int FMHAInferI8CrossCheckArgs(FMHAParamI8 fmha_param, FMHACrossAttnDescriptor desc, const void* q, const void* k,

@@ -55,6 +55,12 @@ constexpr float kBaseScale = 67108864.0f;  // 2^26: float units per integer unit
 constexpr float kBiasOffsetLimit = 4096.0f;  // see the launch code: bound on the exponent offset of the biased path
 constexpr float kLog2Pscale = -7.99995597f;  // log2(128 / 32767): exp2(x + kLog2Pscale) = 128 p / 32767
 constexpr float kLazyLog2 = 10.0f;       // the running O is rescaled only when a row maximum grows by more than this
+// Full-range P (the FULLP variant below): P = rne(255 p) in [0, 255], so |sum of P v| over 128 keys can reach
+// 255 * 127 * 128 = 4145280.  Its GEMM 2 accumulators start at the float 0.1875, which sits exactly 2^22 = 4194304
+// ulps from either end of its binade.
+constexpr float kLog2PscaleFull = -7.00560236f;  // log2(255 / 32767)
+constexpr int kBaseBitsFull = 0x3E400000;
+constexpr float kBaseFull = __builtin_bit_cast(float, kBaseBitsFull);
 
 // FMHA_CHECK_BOUNDS (a test build, never the shipped library): every global access of the kernel is first checked
 // against the tensor - for K and V the head - it belongs to; an access that would leave it is counted in
@@ -125,7 +131,12 @@ __device__ __forceinline__ float half_sum(float x) {
 // and each merge rounds at that magnitude; the host enables it only where that rounding is far below one output LSB.
 // RAGGED: seq_kv is not a multiple of BK.  Everything that serves the partly filled last block is compiled in only
 // then: in the key loop it costs some fifty scalar instructions per block, which the other lengths do not pay.
-template <int D, int BK, bool BIAS, bool FASTACC, bool RAGGED>
+// FULLP: P keeps all 255 steps of a byte, P = rne(255 p) - what the reference plans as "uint8 x int8" (README.md:15,186)
+// and has no code for.  The matrix unit multiplies signed bytes only, so GEMM 2 runs on P - 128 (the byte with its top
+// bit flipped) and the missing 128 * sum_j v[j][c] per key block and output column goes in as the START VALUE of the
+// accumulators: wavefronts 4..7 sum the columns of every V tile one phase before its GEMM 2 (v_dot4 on the transposed
+// operand reads), leave kBaseBitsFull + 128 * sum in LDS, and every wavefront reads its C operand from there.
+template <int D, int BK, bool BIAS, bool FASTACC, bool RAGGED, bool FULLP>
 __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelArgs args) {
   constexpr int kChunks = D / 16;                     // 16-byte chunks per row
   constexpr int kTileBytes = BK * D;                  // one K or V tile
@@ -140,6 +151,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   __shared__ __attribute__((aligned(1024))) int8_t lds[kStages][2][kTileBytes];  // [stage][K|V][tile]; tile j -> stage j % kStages
   __shared__ unsigned char lds_class[kMaxKeyBlocks];  // per key block: bit0 = some key masked, bit1 = all keys masked
   __shared__ unsigned lds_mask[kMaxKeyBlocks * kBlockKSmall / 32];  // bit j%32 of word j/32: key j of this batch entry is masked
+  __shared__ __attribute__((aligned(16))) int lds_colsum[FULLP ? 2 * D : 4];  // FULLP: [key block & 1][output column]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -193,6 +205,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   for (int kk = 0; kk < kDSteps; ++kk)
     k_read_off[kk] = i32 * D + (((2 * kk + g) ^ k_swizzle<D>(i32)) << 4);
   int v_read_off[kDSteps];  // + 32*t*D per key tile, + 16*D for the second half of the operand
+  int colsum_tile, colsum_read_off;
   {
     const int jin = lane & 15, hh = (lane >> 4) & 1;
     const int kslot = jin >> 1;
@@ -200,6 +213,9 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #pragma unroll
     for (int u = 0; u < kDSteps; ++u)
       v_read_off[u] = key_lane * D + (((2 * u + hh) ^ v_swizzle<D>(key_lane)) << 4) + 8 * (jin & 1);
+    // FULLP: wavefront 4 + u sums the columns of output tile u (the same operand reads, a run-time tile index)
+    colsum_tile = wave - 4;
+    colsum_read_off = key_lane * D + (((2 * (colsum_tile & (kDSteps - 1)) + hh) ^ v_swizzle<D>(key_lane)) << 4) + 8 * (jin & 1);
   }
 
   // HBM -> LDS without passing through registers.  Written as inline assembly on purpose: the compiler treats an
@@ -356,6 +372,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   const float bias_c2 = BIAS ? kBase * c2 : 0.f;
   float magic = kMagic;
   asm volatile("" : "+v"(magic));  // a register operand: as a literal it would double the size of every instruction using it
+  int flip_top = (int)0x80808080;
+  if (FULLP) asm volatile("" : "+s"(flip_top));  // a register operand, for the same reason
   v16i base_c = {kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits,
                  kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits};
   asm volatile("" : "+v"(base_c));  // held in registers: as a known constant it is rebuilt by eight moves per key block
@@ -468,7 +486,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       if (!BIAS) off = __builtin_fmaf(fabsf(off), 2.384185791015625e-07f, off);
       if (!BIAS) off = fmaxf(off, args.floor2);
       m_blk = off - bias_c2;
-      const float offq = off - kLog2Pscale;  // exp2(x - offq) = 128 p / 32767: the snorm conversion returns rne(128 p)
+      // exp2(x - offq) = 128 p / 32767: the snorm conversion returns rne(128 p) (FULLP: 255 in place of 128)
+      const float offq = off - (FULLP ? kLog2PscaleFull : kLog2Pscale);
       // Software pipeline over quads of four scores (quad qd = 4 t + a): step s issues the four exponentials of quad s
       // with the four scaling fmas of quad s+1 and the sums and packing of quad s-1 between them.  A wavefront issues in
       // order, a transcendental occupies its unit for about two issue slots, and an instruction that follows one without
@@ -485,10 +504,13 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         const float(&e)[4] = x[qd % 3];
         if (j == 0) s01 = e[0] + e[1];
         if (j == 1) s23 = e[2] + e[3];
-        if (j == 2) lo = __builtin_amdgcn_cvt_pknorm_i16(-e[0], -e[1]);
-        if (j == 3) hi = __builtin_amdgcn_cvt_pknorm_i16(-e[2], -e[3]);
+        if (j == 2) lo = FULLP ? __builtin_amdgcn_cvt_pknorm_i16(e[0], e[1]) : __builtin_amdgcn_cvt_pknorm_i16(-e[0], -e[1]);
+        if (j == 3) hi = FULLP ? __builtin_amdgcn_cvt_pknorm_i16(e[2], e[3]) : __builtin_amdgcn_cvt_pknorm_i16(-e[2], -e[3]);
         if (j == 4) s01 += s23;
-        if (j == 5) pk[qd / 4][qd % 4] = __builtin_amdgcn_perm(__builtin_bit_cast(int, hi), __builtin_bit_cast(int, lo), 0x06040200);
+        if (j == 5) {
+          const int four = __builtin_amdgcn_perm(__builtin_bit_cast(int, hi), __builtin_bit_cast(int, lo), 0x06040200);
+          pk[qd / 4][qd % 4] = FULLP ? four ^ flip_top : four;  // FULLP: the bytes 0..255 become P - 128
+        }
         if (j == 6) l_blk += s01;
       };
       if (kQuads > 0) {
@@ -545,18 +567,32 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     const float take = __builtin_amdgcn_exp2f(m_blk - m_ref);
     l_run = __builtin_fmaf(take, l_blk, l_run);
     if (FASTACC) t_run += take;
-    float neg_take = -take;  // P carries the sign: P = -128 p (inc/fmha_i8.cuh:298)
+    float neg_take = FULLP ? take : -take;  // P carries the sign: P = -128 p (inc/fmha_i8.cuh:298); FULLP: P = 255 p
     asm volatile("" : "+v"(neg_take));  // a plain register operand: as a source modifier it would force the 64-bit encoding
     auto merge_piece = [&](const v16i& oa, int u, int j) {  // four of the sixteen elements of output tile u
 #pragma unroll
       for (int r = 4 * j; r < 4 * j + 4; ++r)
-        o_f[u][r] = __builtin_fmaf(neg_take, FASTACC ? __int_as_float(oa[r]) : __int_as_float(oa[r]) - kBase, o_f[u][r]);
+        o_f[u][r] = __builtin_fmaf(neg_take, FASTACC ? __int_as_float(oa[r]) : __int_as_float(oa[r]) - (FULLP ? kBaseFull : kBase),
+                                   o_f[u][r]);
     };
 
     const int8_t* lds_v = &lds[kb & (kStages - 1)][1][0];
     typedef v2i __attribute__((address_space(3))) * lds_v2i_ptr;
     v2i va[2][kKeyTiles][2];  // transposed V operands of one output tile (all key tiles), one output tile ahead
-    v16i oacc[2];
+    // FULLP: the accumulators of tile u start at what wavefronts 4..7 left in LDS for this key block (four 128-bit
+    // reads per tile, fetched one tile ahead like the operands: a third buffer, since tile u-1 is still being merged)
+    constexpr int kOaccBufs = FULLP ? 3 : 2;
+    v16i oacc[kOaccBufs];
+    auto ob = [&](int u) { return FULLP ? u % 3 : u & 1; };
+    auto read_start = [&](int u) {
+      const int* cs = &lds_colsum[(kb & 1) * D + 32 * u + 4 * g];
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const v4i w = *reinterpret_cast<const v4i*>(cs + 8 * a);
+#pragma unroll
+        for (int bb = 0; bb < 4; ++bb) oacc[ob(u)][4 * a + bb] = w[bb];
+      }
+    };
     auto read_tile = [&](int u) {
 #pragma unroll
       for (int t = 0; t < kKeyTiles; ++t) {
@@ -565,19 +601,23 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
             __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u] + 32 * t * D + 16 * D));
       }
     };
+    if (FULLP) read_start(0);
     read_tile(0);
 #pragma unroll
     for (int u = 0; u < kDSteps; ++u) {
-      if (u + 1 < kDSteps) read_tile(u + 1);
+      if (u + 1 < kDSteps) {
+        read_tile(u + 1);
+        if (FULLP) read_start(u + 1);
+      }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int t = 0; t < kKeyTiles; ++t) {
         const v4i a = {va[u & 1][t][0][0], va[u & 1][t][0][1], va[u & 1][t][1][0], va[u & 1][t][1][1]};
-        oacc[u & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, pk[t], t == 0 ? base_c : oacc[u & 1], 0, 0, 0);
+        oacc[ob(u)] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, pk[t], (t == 0 && !FULLP) ? base_c : oacc[ob(u)], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         if (u >= 1) {
 #pragma unroll
-          for (int j = t * 4 / kKeyTiles; j < (t + 1) * 4 / kKeyTiles; ++j) merge_piece(oacc[(u - 1) & 1], u - 1, j);
+          for (int j = t * 4 / kKeyTiles; j < (t + 1) * 4 / kKeyTiles; ++j) merge_piece(oacc[ob(u - 1)], u - 1, j);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -588,8 +628,31 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       }
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) merge_piece(oacc[(kDSteps - 1) & 1], kDSteps - 1, j);
+    for (int j = 0; j < 4; ++j) merge_piece(oacc[ob(kDSteps - 1)], kDSteps - 1, j);
   };
+  // FULLP, wavefronts 4..7 (wavefront 4 + u: output tile u): the start values of GEMM 2 of key block kb.  The operand
+  // reads of GEMM 2 hand lane (i32, g) sixteen keys of column 32u + i32 per key tile; v_dot4 against four ones sums
+  // them, the two halves of the wavefront add up to the whole tile.  Rows of a tile that stand for keys which do not
+  // exist (a ragged end) are counted like any other: their P is 0, i.e. the byte -128, and the two cancel.
+  auto phase_colsum = [&](int kb) {
+    if (colsum_tile >= 0 && colsum_tile < kDSteps) {
+      const int8_t* lds_v = &lds[kb & (kStages - 1)][1][0];
+      typedef v2i __attribute__((address_space(3))) * lds_v2i_ptr;
+      int sum = 0;
+#pragma unroll
+      for (int t = 0; t < kKeyTiles; ++t)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const v2i w = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + colsum_read_off + 32 * t * D + 16 * D * h));
+          sum = __builtin_amdgcn_sdot4(w[0], 0x01010101, sum, false);
+          sum = __builtin_amdgcn_sdot4(w[1], 0x01010101, sum, false);
+        }
+      const auto r = __builtin_amdgcn_permlane32_swap(sum, sum, false, false);
+      lds_colsum[(kb & 1) * D + 32 * colsum_tile + i32] = kBaseBitsFull + 128 * ((int)r[0] + (int)r[1]);
+    }
+  };
+  // An LDS write is not waited for by the hand-written barrier: wavefronts 4..7 do so at the end of the phase.
+  auto colsum_written = [&]() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
 
   // ---- the tick schedule -------------------------------------------------------------------------------------------
   // A tick is the interval between two workgroup barriers.  Every key block i is two phases per wavefront: an MFMA
@@ -627,6 +690,11 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // have just done so), the pair of this one.
   auto wait_tiles = [&](bool issued_after_softmax) { wait_all_but(!kLoadsInMfmaPhase && issued_after_softmax ? 4 : 2); };
   auto issue_after_softmax = [&](int i) { if (!kLoadsInMfmaPhase) issue_for(i); };
+  // FULLP: V(m) is summed by wavefronts 4..7 in tick 2m+1, one tick before its GEMM 2, so it is barrier 2m+1 that
+  // publishes it.  Wavefronts 0..3 arrive there from their MFMA phase (the pair issued last may stay in flight),
+  // wavefronts 4..7 from their softmax (the pair they have just issued; none where the loads go out in the MFMA phase).
+  auto wait_v_for_colsum_a = [&]() { if (FULLP) wait_all_but(2); };
+  auto wait_v_for_colsum_b = [&]() { if (FULLP) wait_all_but(kLoadsInMfmaPhase ? 0 : 2); };
   auto issue_in_mfma_phase = [&](int i) { if (kLoadsInMfmaPhase) issue_for(i); };
   v16i acc[kKeyTiles];  // S^T of the block whose softmax comes next (GEMM 1 -> softmax, across a barrier)
   int mx[2];
@@ -653,6 +721,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     if (active) {
       for (; i + 1 < n && i + 1 < kb_plain; ++i) {
         v4i pk[kKeyTiles];
+        wait_v_for_colsum_a();
         barrier();
         phase_softmax(i, 0, acc, pk, mx);
         issue_after_softmax(i);
@@ -668,6 +737,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       const int cls = cls_of(i);
       const bool work = active && !(cls & 2);
       v4i pk[kKeyTiles];
+      wait_v_for_colsum_a();
       barrier();                               // barrier 2i+1
       if (work) phase_softmax(i, cls, acc, pk, mx);
       issue_after_softmax(i);
@@ -683,9 +753,12 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     barrier();                                 // barrier 2n+1: wavefronts 4..7 run their last MFMA phase after it
   } else {
     issue_first();
+    if (FULLP) wait_all_but(3);                // V(0) has landed: K1 K2 V1 may be in flight
     barrier();                                 // barrier 1
+    if (FULLP && n > 0) phase_colsum(0);
     if (n > 0 && works(0)) phase_gemm1(0, acc, mx);
     else forget_scores();
+    if (FULLP) colsum_written();
     int i = 0;
     if (active) {  // steady state, see above
       for (; i + 1 < n && i + 1 < kb_plain; ++i) {
@@ -694,10 +767,13 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         barrier();
         phase_softmax(i, 0, acc, pk, mx);
         issue_after_softmax(i);
+        wait_v_for_colsum_b();
         barrier();
         raise_priority();
         phase_gemm2_merge(i, pk, min(i + 3, last), min(i + 2, last));
+        if (FULLP) phase_colsum(i + 1);
         phase_gemm1(i + 1, acc, mx);
+        if (FULLP) colsum_written();
         drop_priority();
       }
     }
@@ -709,12 +785,15 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       barrier();                               // barrier 2i+2
       if (work) phase_softmax(i, cls, acc, pk, mx);
       issue_after_softmax(i);
+      wait_v_for_colsum_b();
       barrier();                               // barrier 2i+3
       raise_priority();
       if (work) phase_gemm2_merge(i, pk, min(i + 3, last), min(i + 2, last));
       else issue_in_mfma_phase(i);
+      if (FULLP && i + 1 < n) phase_colsum(i + 1);
       if (i + 1 < n && works(i + 1)) phase_gemm1(i + 1, acc, mx);
       else forget_scores();
+      if (FULLP) colsum_written();
       drop_priority();
     }
   }
@@ -724,7 +803,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // ---- epilogue: normalise, requantise, store (inc/fmha_i8.cuh:318-332) --------------------------------------------
   // l_run sums 128 p / 32767 and O sums 128 p v, so mean(v) = O / (32767 l_run); a row with no unmasked key yields 0
   const float fin = (l_run > 0.f) ? args.out_scale * (128.f / kSnorm) * kBaseScale / l_run : 0.f;
-  const float corr = FASTACC ? kBase * t_run : 0.f;
+  const float corr = FASTACC ? (FULLP ? -kBaseFull * t_run : kBase * t_run) : 0.f;
   int w[kDSteps][4];  // w[u][a]: the four int8 of output dims 32u + 8a + 4g .. +3 of query row i32
 #pragma unroll
   for (int u = 0; u < kDSteps; ++u)

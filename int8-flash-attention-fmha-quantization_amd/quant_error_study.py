@@ -13,9 +13,11 @@ simulates:
                (inc/fmha_i8.cuh:181-253,298-315)
   block_local_full
                the same with 255 steps: the "uint8 x int8" variant the reference plans (README.md:15,186), which on
-               int8 matrix hardware would be P - 128 as int8 plus 128 times the column sums of V per block
+               int8 matrix hardware is P - 128 as int8 plus 128 times the column sums of V per block
   kernel       (optional, --kernel) the HIP kernel itself through libfmha_i8.so, int8 output de-quantised with
                o_amax = max |float O|; adds the output quantisation on top of block_local; multiples of 64 only
+  kernel_full  (with --kernel) the kernel's 255-step entry point, FMHAInferI8CrossFullRangeP: block_local_full plus
+               the output quantisation
 
 Everything else follows the scripts: Q, K, V standard normal, [S, d] (one head), symmetric int8 quantisation of Q, K, V
 by abs-max with numpy's round-half-even, int32 Q.K^T, float softmax, P quantised to --levels steps, int32 P.V,
@@ -110,6 +112,7 @@ def simulate(seq_len, head_dim, rng, kernel=None, levels=SOFTMAX_QUANT_SCALE):
     out.update(q=i8_q, k=i8_k, v=i8_v, q_amax=q_amax, k_amax=k_amax, v_amax=v_amax, o_amax=o_amax)
     if kernel is not None and seq_len % 64 == 0:
         out["kernel"] = kernel(i8_q, i8_k, i8_v, q_amax, k_amax, v_amax, o_amax)
+        out["kernel_full"] = kernel(i8_q, i8_k, i8_v, q_amax, k_amax, v_amax, o_amax, full_range_p=True)
     return out
 
 
@@ -139,10 +142,10 @@ def hip_kernel_runner():
         raise RuntimeError("--kernel needs a GPU")
     dev = torch.device("cuda:0")
 
-    def run(q, k, v, q_amax, k_amax, v_amax, o_amax):
+    def run(q, k, v, q_amax, k_amax, v_amax, o_amax, full_range_p=False):
         t = [torch.from_numpy(np.ascontiguousarray(a[None, None])).to(dev) for a in (q, k, v)]
         mask = torch.zeros((1, k.shape[0]), dtype=torch.int8, device=dev)
-        o = pkg.fmha_infer_i8(t[0], t[1], t[2], mask, q_amax, k_amax, v_amax, o_amax)
+        o = pkg.fmha_infer_i8(t[0], t[1], t[2], mask, q_amax, k_amax, v_amax, o_amax, full_range_p=full_range_p)
         torch.cuda.synchronize()
         return o[0, 0].cpu().numpy().astype(f32) / f32(127.0) * f32(o_amax)  # inc/utils.hpp:53
 
@@ -151,7 +154,7 @@ def hip_kernel_runner():
 
 def table_seqlen(lengths, head_dim, seed, kernel=None, levels=SOFTMAX_QUANT_SCALE):
     """Rows (seq_len, sum |error| per scheme): what fmha_i8_quant_error_seqlen.py:119-130 plots."""
-    cols = SCHEMES + (("kernel",) if kernel is not None else ())
+    cols = SCHEMES + (("kernel", "kernel_full") if kernel is not None else ())
     rows = []
     for S in lengths:
         r = simulate(S, head_dim, np.random.default_rng([seed, S, head_dim]), kernel, levels)
@@ -161,7 +164,7 @@ def table_seqlen(lengths, head_dim, seed, kernel=None, levels=SOFTMAX_QUANT_SCAL
 
 def table_deviation(seq_len, head_dim, seed, kernel=None, levels=SOFTMAX_QUANT_SCALE):
     """Rows (token, relative L2 deviation per scheme): what fmha_i8_quant_deviation.py:75-126 plots."""
-    cols = SCHEMES + (("kernel",) if kernel is not None else ())
+    cols = SCHEMES + (("kernel", "kernel_full") if kernel is not None else ())
     r = simulate(seq_len, head_dim, np.random.default_rng([seed, seq_len, head_dim]), kernel, levels)
     dev = [row_deviation(r[c], r["ref"]) for c in cols if c in r]
     return ("token",) + tuple(c for c in cols if c in r), [[i] + [float(d[i]) for d in dev] for i in range(seq_len)]

@@ -160,10 +160,13 @@ inline void parallel_for(long n, int threads, F&& body) {
 //   * a row with no unmasked key at all yields 0 (as inc/cpuSoftmax.hpp:18-47 does).
 inline void fmha_i8_head_blockwise(const int8_t* q, const int8_t* k, const int8_t* v, const int8_t* mask, int8_t* o,
                                    int Sq, int S, int d, float q_amax, float k_amax, float v_amax, float o_amax,
-                                   int block) {
+                                   int block, bool full_range_p = false) {
   const float row_scale = reference_row_scale(d);                    // fmha_i8.cuh:71
   const float scale_qk_out = q_amax * k_amax / (127.f * 127.f);      // fmha_i8.cuh:72
-  const float scale_v_out = v_amax * (1.0f / (o_amax * 128.f));      // fmha_i8.cuh:318
+  // full_range_p: the "uint8 x int8" variant that the reference plans and does not have (README.md:15,186): P keeps
+  // all 255 steps of a byte, P = rne(255 p) in [0, 255], and every 128 of the pipeline becomes 255.
+  const float p_scale = full_range_p ? 255.f : -128.f;               // fmha_i8.cuh:241
+  const float scale_v_out = v_amax * (1.0f / (o_amax * std::fabs(p_scale)));  // fmha_i8.cuh:318
   const int kMaskedInt = static_cast<int>(-1e6);                     // fmha_i8.cuh:191-192
   std::vector<int32_t> s_int(block);
   std::vector<float> p_f(block);
@@ -200,9 +203,10 @@ inline void fmha_i8_head_blockwise(const int8_t* q, const int8_t* k, const int8_
         p_f[j] = mask[k0 + j] ? 0.0f : e;
         l_blk += p_f[j];
       }
-      // P -> int8 in [-128, 0], round-half-even (fmha_i8.cuh:241,249).
+      // P -> int8 in [-128, 0], round-half-even (fmha_i8.cuh:241,249); full range: a byte in [0, 255].
       for (int j = 0; j < nb; ++j)
-        p_i8[j] = (int32_t)std::nearbyint(std::max(std::min(-128.f * p_f[j], 0.f), -128.f));
+        p_i8[j] = full_range_p ? (int32_t)std::nearbyint(std::max(std::min(255.f * p_f[j], 255.f), 0.f))
+                               : (int32_t)std::nearbyint(std::max(std::min(-128.f * p_f[j], 0.f), -128.f));
       // GEMM 2 (fmha_i8.cuh:255-296): exact int32.
       std::fill(o_tilde.begin(), o_tilde.end(), 0);
       for (int j = 0; j < nb; ++j) {
@@ -218,7 +222,8 @@ inline void fmha_i8_head_blockwise(const int8_t* q, const int8_t* k, const int8_
       const float l_new = a * l_old + bb * l_blk;
       const float inv = 1.0f / l_new;
       const float keep = l_old * a;
-      for (int c = 0; c < d; ++c) o_f[c] = inv * (keep * o_f[c] + bb * (-1.f * static_cast<float>(o_tilde[c])));
+      const float p_sign = full_range_p ? 1.f : -1.f;
+      for (int c = 0; c < d; ++c) o_f[c] = inv * (keep * o_f[c] + bb * (p_sign * static_cast<float>(o_tilde[c])));
       l_old = l_new;
       m_old = m_new;
     }
@@ -236,7 +241,7 @@ inline void fmha_i8_head_blockwise(const int8_t* q, const int8_t* k, const int8_
 inline void fmha_i8_cpu_blockwise_cross(const int8_t* q, const int8_t* k, const int8_t* v, const int8_t* mask,
                                         int8_t* o, int B, int H, int Sq, int S, int d, float q_amax, float k_amax,
                                         float v_amax, float o_amax, int block, int threads, long head_begin,
-                                        long head_end) {
+                                        long head_end, bool full_range_p = false) {
   const long hd_q = (long)Sq * d, hd = (long)S * d;
   head_begin = std::max<long>(head_begin, 0);
   head_end = std::min<long>(head_end, (long)B * H);
@@ -244,7 +249,7 @@ inline void fmha_i8_cpu_blockwise_cross(const int8_t* q, const int8_t* k, const 
     const long bh = head_begin + t;
     const long b = bh / H;
     fmha_i8_head_blockwise(q + bh * hd_q, k + bh * hd, v + bh * hd, mask + b * S, o + bh * hd_q, Sq, S, d, q_amax,
-                           k_amax, v_amax, o_amax, block);
+                           k_amax, v_amax, o_amax, block, full_range_p);
   });
 }
 inline void fmha_i8_cpu_blockwise(const int8_t* q, const int8_t* k, const int8_t* v, const int8_t* mask, int8_t* o,

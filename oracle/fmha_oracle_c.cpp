@@ -47,6 +47,14 @@ void oracle_fmha_i8_blockwise_cross(const int8_t* q, const int8_t* k, const int8
   fmha_i8_cpu_blockwise_cross(q, k, v, mask, o, B, H, Sq, S, d, q_amax, k_amax, v_amax, o_amax, block, threads,
                               head_begin, head_end);
 }
+// ... and with P on all 255 steps of a byte (README.md:15,186 plans it as "uint8 x int8"; the reference has no code for it).
+void oracle_fmha_i8_blockwise_cross_full_range_p(const int8_t* q, const int8_t* k, const int8_t* v, const int8_t* mask,
+                                                 int8_t* o, int B, int H, int Sq, int S, int d, float q_amax,
+                                                 float k_amax, float v_amax, float o_amax, int block, int threads,
+                                                 long head_begin, long head_end) {
+  fmha_i8_cpu_blockwise_cross(q, k, v, mask, o, B, H, Sq, S, d, q_amax, k_amax, v_amax, o_amax, block, threads,
+                              head_begin, head_end, true);
+}
 // test_fmha_i8.cpp:141-162 float path.
 void oracle_fmha_fp32(const float* q, const float* k, const float* v, const int8_t* mask, float* o, int B, int H, int S,
                       int d, int threads, long head_begin, long head_end) {

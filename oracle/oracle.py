@@ -55,6 +55,8 @@ def lib():
                                                      C.c_int, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int,
                                                      C.c_int, C.c_long, C.c_long]
         L.oracle_fmha_i8_blockwise_cross.restype = None
+        L.oracle_fmha_i8_blockwise_cross_full_range_p.argtypes = L.oracle_fmha_i8_blockwise_cross.argtypes
+        L.oracle_fmha_i8_blockwise_cross_full_range_p.restype = None
         L.oracle_fmha_fp32.argtypes = [_f32p, _f32p, _f32p, _i8p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
                                        C.c_long, C.c_long]
         L.oracle_hardware_threads.restype = C.c_int
@@ -146,21 +148,21 @@ def fmha_i8_blockwise(q, k, v, mask, q_amax, k_amax, v_amax, o_amax, block=128, 
     return o
 
 
-def fmha_i8_blockwise_cross(q, k, v, mask, q_amax, k_amax, v_amax, o_amax, block=None, threads=None):
+def fmha_i8_blockwise_cross(q, k, v, mask, q_amax, k_amax, v_amax, o_amax, block=None, threads=None,
+                            full_range_p=False):
     """q: int8 [B,H,Sq,d]; k, v: int8 [B,H,S,d]; mask: int8 [B,S], nonzero = masked out.  Returns int8 O [B,H,Sq,d].
     block defaults to what the reference's ladder would give S: 128 keys for multiples of 128, else 64.  A key count
-    that is no multiple of 64 means the next multiple of 64 with the missing keys masked out."""
+    that is no multiple of 64 means the next multiple of 64 with the missing keys masked out.
+    full_range_p: P = rne(255 p) in [0, 255] instead of rne(-128 p) in [-128, 0] (README.md:15,186, planned there)."""
     B, H, Sq, d = q.shape
     S = k.shape[2]
     assert k.shape == (B, H, S, d) and v.shape == k.shape and mask.shape == (B, S)
     q, k, v = (np.ascontiguousarray(t, dtype=np.int8) for t in (q, k, v))
     mask = np.ascontiguousarray(mask, dtype=np.int8)
     o = np.zeros_like(q)
-    lib().oracle_fmha_i8_blockwise_cross(q.reshape(-1), k.reshape(-1), v.reshape(-1), mask.reshape(-1), o.reshape(-1),
-                                         B, H, Sq, S, d, q_amax, k_amax, v_amax, o_amax,
-                                         block or (128 if (S + 63) // 64 * 64 % 128 == 0 else 64),
-                                         threads or hardware_threads(),
-                                         0, B * H)
+    fn = lib().oracle_fmha_i8_blockwise_cross_full_range_p if full_range_p else lib().oracle_fmha_i8_blockwise_cross
+    fn(q.reshape(-1), k.reshape(-1), v.reshape(-1), mask.reshape(-1), o.reshape(-1), B, H, Sq, S, d, q_amax, k_amax,
+       v_amax, o_amax, block or (128 if (S + 63) // 64 * 64 % 128 == 0 else 64), threads or hardware_threads(), 0, B * H)
     return o
 
 

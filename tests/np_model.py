@@ -7,11 +7,12 @@ import numpy as np
 f32 = np.float32
 
 
-def fmha_i8_head(q, k, v, mask, q_amax, k_amax, v_amax, o_amax, block=128):
+def fmha_i8_head(q, k, v, mask, q_amax, k_amax, v_amax, o_amax, block=128, full_range_p=False):
+    """full_range_p: P = rne(255 p) in [0, 255] (the variant README.md:15,186 plans) instead of rne(-128 p)."""
     S, d = q.shape
     row_scale = f32(1.0) / f32(np.sqrt(f32(d)))
     scale_qk = f32(q_amax) * f32(k_amax) / (f32(127.0) * f32(127.0))
-    scale_v = f32(v_amax) * (f32(1.0) / (f32(o_amax) * f32(128.0)))
+    scale_v = f32(v_amax) * (f32(1.0) / (f32(o_amax) * f32(255.0 if full_range_p else 128.0)))
     qi = q.astype(np.int32)
     m_run = np.full(S, -1e6, f32)
     l_run = np.zeros(S, f32)
@@ -26,7 +27,10 @@ def fmha_i8_head(q, k, v, mask, q_amax, k_amax, v_amax, o_amax, block=128):
         x = ((row_scale * s_int.astype(f32)).astype(f32) * scale_qk).astype(f32) - m_blk[:, None]
         p = np.where(mk[None, :], f32(0), np.exp(x.astype(f32))).astype(f32)
         l_blk = p.sum(axis=1, dtype=f32)
-        p_i8 = np.rint(np.clip(f32(-128.0) * p, -128, 0)).astype(np.int32)  # np.rint rounds half to even
+        if full_range_p:
+            p_i8 = -np.rint(np.clip(f32(255.0) * p, 0, 255)).astype(np.int32)  # (negated: the merge below subtracts)
+        else:
+            p_i8 = np.rint(np.clip(f32(-128.0) * p, -128, 0)).astype(np.int32)  # np.rint rounds half to even
         o_tilde = p_i8 @ v[k0:k0 + block].astype(np.int32)  # [S, d] exact
         m_new = np.maximum(m_run, m_blk)
         a = np.exp((m_run - m_new).astype(f32)).astype(f32)
@@ -39,12 +43,13 @@ def fmha_i8_head(q, k, v, mask, q_amax, k_amax, v_amax, o_amax, block=128):
     return out
 
 
-def fmha_i8(q, k, v, mask, q_amax, k_amax, v_amax, o_amax, block=128):
+def fmha_i8(q, k, v, mask, q_amax, k_amax, v_amax, o_amax, block=128, full_range_p=False):
     B, H, S, d = q.shape
     o = np.zeros_like(q)
     for b in range(B):
         for h in range(H):
-            o[b, h] = fmha_i8_head(q[b, h], k[b, h], v[b, h], mask[b], q_amax, k_amax, v_amax, o_amax, block)
+            o[b, h] = fmha_i8_head(q[b, h], k[b, h], v[b, h], mask[b], q_amax, k_amax, v_amax, o_amax, block,
+                                   full_range_p)
     return o
 
 

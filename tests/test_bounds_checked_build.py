@@ -31,13 +31,14 @@ def checked(pkg):
     return lib
 
 
-def _run(pkg, lib, dev, q, k, v, mask, scales):
+def _run(pkg, lib, dev, q, k, v, mask, scales, full_range_p=False):
     import torch
     t = [torch.from_numpy(np.ascontiguousarray(a)).to(dev) for a in (q, k, v, mask)]
     o = torch.empty_like(t[0])
     B, H, Sq, d = q.shape
-    st = lib.FMHAInferI8Cross(None, pkg.FMHAParamI8(*scales, 1.0), pkg.FMHACrossAttnDescriptor(B, Sq, k.shape[2], H, d),
-                              *(x.data_ptr() for x in t), o.data_ptr())
+    entry = lib.FMHAInferI8CrossFullRangeP if full_range_p else lib.FMHAInferI8Cross
+    st = entry(None, pkg.FMHAParamI8(*scales, 1.0), pkg.FMHACrossAttnDescriptor(B, Sq, k.shape[2], H, d),
+               *(x.data_ptr() for x in t), o.data_ptr())
     assert st == pkg.FMHA_I8_OK
     return o
 
@@ -62,7 +63,8 @@ def test_checked_build_counts_nothing_on_any_shape(pkg, orc, checked, dev):
         q = fc.make_inputs(B, H, Sq, d, seed=700 + n)["q"]
         scales = (c["q_amax"], c["k_amax"], c["v_amax"], 1.0)
         print("shape", B, H, Sq, S, d, flush=True)
-        o = _run(pkg, checked, dev, q, k, v, mask, scales)
-        assert checked.FMHAInferI8DebugOutOfBounds() == 0, (B, H, Sq, S, d)
-        st = fc.parity_stats(o.cpu().numpy(), orc.fmha_i8_blockwise_cross(q, k, v, mask, *scales))
-        assert st["within1"] >= 0.999 and st["max"] <= 2, ((B, H, Sq, S, d), st)
+        for full in (False, True):  # the reference's P on 128 steps, and P on 255 steps
+            o = _run(pkg, checked, dev, q, k, v, mask, scales, full)
+            assert checked.FMHAInferI8DebugOutOfBounds() == 0, (B, H, Sq, S, d, full)
+            st = fc.parity_stats(o.cpu().numpy(), orc.fmha_i8_blockwise_cross(q, k, v, mask, *scales, full_range_p=full))
+            assert st["within1"] >= 0.999 and st["max"] <= 2, ((B, H, Sq, S, d, full), st)

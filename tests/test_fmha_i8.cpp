@@ -9,6 +9,7 @@
 //                                           uniform(+-0.5) Q/K, |uniform| V, scattered 20 % mask, o_amax measured
 //   test_fmha_i8 --B 2 --H 4 --S 512 --d 64 [--valid L | --pad none|bert|tail16th|scatter] [--dist normal|student_t|reference]
 //   ... --Sq 100                            that many query rows per head over the S keys (FMHAInferI8Cross)
+//   ... --full-range-p                      P on 255 steps (FMHAInferI8CrossFullRangeP), checked against that mode of the checker
 //   common: --seed N --iters N --warmup N --cpu-heads N (0 = all) --cpu-threads N --json FILE --no-check
 //   --quant MiB            instead of attention cases: abs-max, quantise and de-quantise (include/fmha_quant.h) over that
 //                          many MiB of fp32 input, checked bit for bit against the CPU checker and timed against HBM
@@ -93,6 +94,7 @@ struct Options {
   long cpu_heads = 8;
   int cpu_threads = 0;
   bool check = true;
+  bool full_range_p = false;
   std::string json;
 };
 
@@ -150,11 +152,14 @@ double seconds_since(std::chrono::steady_clock::time_point t0) {
 }
 
 bool run_case(const Case& c, const Options& opt, FILE* json) {
-  const bool cross = c.Sq > 0 && c.Sq != c.S;  // queries and keys differ in number: FMHAInferI8Cross
-  const int Sq = cross ? c.Sq : c.S;
+  const bool full = opt.full_range_p;
+  const bool cross = full || (c.Sq > 0 && c.Sq != c.S);  // queries and keys differ in number: FMHAInferI8Cross
+  const int Sq = c.Sq > 0 ? c.Sq : c.S;
+  const bool square = Sq == c.S;  // the reference's float path and its acceptance metric apply
   printf("compute type=int32, data type=int8, batch_num=%d, seq_len=%d, head_num=%d, head_dim=%d, dist=%s, pad=%s",
          c.B, c.S, c.H, c.d, c.dist.c_str(), c.pad.c_str());
   if (cross) printf(", query rows=%d", Sq);
+  if (full) printf(", P on 255 steps");
   printf("\n");
   fflush(stdout);
   Data t = generate(c, opt.seed);
@@ -166,7 +171,7 @@ bool run_case(const Case& c, const Options& opt, FILE* json) {
   std::vector<float> o_ref(nq, 0.f);
   float o_amax = 1.0f;
   double cpu_fp32_s = 0, cpu_i8_s = 0;
-  if (opt.check && !cross) {  // (the reference's float path is square: S queries over S keys)
+  if (opt.check && square) {  // (the reference's float path is square: S queries over S keys)
     auto t0 = std::chrono::steady_clock::now();
     fmha_oracle::fmha_fp32_cpu(t.qf.data(), t.kf.data(), t.vf.data(), t.mask.data(), o_ref.data(), c.B, c.H, c.S, c.d,
                                threads, 0, cpu_heads);
@@ -195,11 +200,13 @@ bool run_case(const Case& c, const Options& opt, FILE* json) {
   FMHACrossAttnDescriptor xdesc;
   xdesc.batch_num = c.B, xdesc.seq_len_q = Sq, xdesc.seq_len_kv = c.S, xdesc.head_num = c.H, xdesc.head_dim = c.d;
   auto call = [&]() {
-    if (cross) (void)FMHAInferI8Cross(stream, param, xdesc, dq, dk, dv, dm, dout);
+    if (full) (void)FMHAInferI8CrossFullRangeP(stream, param, xdesc, dq, dk, dv, dm, dout);
+    else if (cross) (void)FMHAInferI8Cross(stream, param, xdesc, dq, dk, dv, dm, dout);
     else gpuImpl::FMHAInferI8(stream, param, desc, dq, dk, dv, dm, dout, true);
   };
-  const int st = cross ? FMHAInferI8Cross(stream, param, xdesc, dq, dk, dv, dm, dout)
-                       : FMHAInferI8Status(stream, param, desc, dq, dk, dv, dm, dout, true);  // warm-up, checked
+  const int st = full    ? FMHAInferI8CrossFullRangeP(stream, param, xdesc, dq, dk, dv, dm, dout)
+                 : cross ? FMHAInferI8Cross(stream, param, xdesc, dq, dk, dv, dm, dout)
+                         : FMHAInferI8Status(stream, param, desc, dq, dk, dv, dm, dout, true);  // warm-up, checked
   if (st != FMHA_I8_OK) {
     fprintf(stderr, "launch failed: %s\n", FMHAInferI8StatusString(st));
     return false;
@@ -248,7 +255,7 @@ bool run_case(const Case& c, const Options& opt, FILE* json) {
     auto t0 = std::chrono::steady_clock::now();
     fmha_oracle::fmha_i8_cpu_blockwise_cross(t.q.data(), t.k.data(), t.v.data(), t.mask.data(), want.data(), c.B, c.H,
                                              Sq, c.S, c.d, t.q_amax, t.k_amax, t.v_amax, o_amax,
-                                             (c.S + 63) / 64 * 64 % 128 == 0 ? 128 : 64, threads, 0, cpu_heads);
+                                             (c.S + 63) / 64 * 64 % 128 == 0 ? 128 : 64, threads, 0, cpu_heads, full);
     cpu_i8_s = seconds_since(t0);
     const long m = cpu_heads * Sq * c.d;
     int worst = 0;
@@ -258,12 +265,12 @@ bool run_case(const Case& c, const Options& opt, FILE* json) {
       worst = std::max(worst, dl);
     }
     const double within1 = (double)(hist[0] + hist[1]) / m;
-    if (!cross) dev_pct = fmha_oracle::mean_rel_deviation_pct(o.data(), o_ref.data(), m, o_amax);  // inc/utils.hpp:59-89
-    pass = within1 >= 0.999 && worst <= 2 && (cross || !c.measured_o_amax || dev_pct < 20.f);
+    if (square) dev_pct = fmha_oracle::mean_rel_deviation_pct(o.data(), o_ref.data(), m, o_amax);  // inc/utils.hpp:59-89
+    pass = within1 >= 0.999 && worst <= 2 && (!square || !c.measured_o_amax || dev_pct < 20.f);
     printf("parity vs int8 CPU checker on %ld of %ld heads: delta 0: %ld, 1: %ld, 2: %ld, >2: %ld -> within 1 LSB "
            "%.5f, max %d  [%s]\n", cpu_heads, heads, hist[0], hist[1], hist[2], hist[3], within1, worst,
            pass ? "PASS" : "FAIL");
-    if (!cross)
+    if (square)
       printf("INT8 average absolute deviation vs float path: %f %%%s\n", dev_pct,
              c.measured_o_amax ? " (reference criterion: < 20)" : " (o_amax fixed at 1: reported only)");
     printf("CPU: float path %.3f s, int8 checker %.3f s, %ld heads, %d threads\n", cpu_fp32_s, cpu_i8_s, cpu_heads,
@@ -421,6 +428,7 @@ int main(int argc, char** argv) {
     else if (a == "--cpu-heads") opt.cpu_heads = atol(val());
     else if (a == "--cpu-threads") opt.cpu_threads = atoi(val());
     else if (a == "--no-check") opt.check = false;
+    else if (a == "--full-range-p") opt.full_range_p = true;
     else if (a == "--json") opt.json = val();
     else if (a == "--calibrate-copy") calib_mib = atol(val());
     else if (a == "--quant") quant_mib = atol(val());

@@ -32,7 +32,7 @@ def test_no_read_of_an_asynchronously_loaded_register_before_its_wait(tmp_path):
                     "-packed-fp32-ops", "-S", "--cuda-device-only", "-o", out, SRC], check=True, capture_output=True)
     text = open(out).read()
     funcs = re.split(r"\n(?=_ZN14fmha_i8_gfx95018fmha_i8_fwd_kernel[^\n]*:\s)", text)[1:]
-    assert len(funcs) == 32
+    assert len(funcs) == 64
     checked = 0
     for f in funcs:
         name = f.split(":")[0]
