@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the INT8 fused attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--no-cpu-baseline] [--full-range-p]
 
 One "step" is one FMHAInferI8 call (through the C ABI of libfmha_i8.so) on one synthetic batch that is already
 resident in HBM.  The default warm-up is 2000 calls (about 60 ms): the shader clock needs some 40 ms of load to settle,
@@ -76,6 +76,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2000)
     ap.add_argument("--workload", default="C3", choices=["C1", "C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--full-range-p", action="store_true", help="time FMHAInferI8CrossFullRangeP (P on 255 steps) "
+                    "instead of the reference's entry point; not the headline configuration")
     ap.add_argument("--cpu-heads", type=int, default=64, help="heads in the CPU-baseline sample")
     ap.add_argument("--cpu-threads", type=int, default=16)
     args = ap.parse_args()
@@ -104,8 +106,14 @@ def main():
     lib = pkg.load_library()
     call_args = (stream.cuda_stream, P, A, q.data_ptr(), k.data_ptr(), v.data_ptr(), m.data_ptr(), o.data_ptr(), True)
 
+    entry = lib.FMHAInferI8Status
+    if args.full_range_p:
+        entry = lib.FMHAInferI8CrossFullRangeP
+        call_args = (stream.cuda_stream, P, pkg.FMHACrossAttnDescriptor(B, S, S, H, d), q.data_ptr(), k.data_ptr(),
+                     v.data_ptr(), m.data_ptr(), o.data_ptr())
+
     def step():  # the C entry point itself, pointers bound once: the host side must not be what is measured
-        st = lib.FMHAInferI8Status(*call_args)
+        st = entry(*call_args)
         if st != 0:
             raise pkg.FMHAError(st, pkg.status_string(st))
 
@@ -136,22 +144,30 @@ def main():
         "pct_of_int8_peak": 100.0 * tops / INT8_PEAK_TOPS,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": "%s: B=%d H=%d S=%d d=%d int8 Q/K/V from %s with per-tensor amax, o_amax=1, "
-                               "%d of %d keys valid, mask polarity nonzero=masked-out" %
-                               (args.workload, B, H, S, d, fc.CONFIGS[args.workload]["dist"], int(valid.sum()), B * S),
+                               "%d of %d keys valid, mask polarity nonzero=masked-out%s" %
+                               (args.workload, B, H, S, d, fc.CONFIGS[args.workload]["dist"], int(valid.sum()), B * S,
+                                ", P on 255 steps (FMHAInferI8CrossFullRangeP)" if args.full_range_p else ""),
                    "batch_num": B, "head_num": H, "seq_len": S, "head_dim": d, "ops_per_call": ops,
                    "ops_per_call_unmasked_keys_only": ops_unmasked,
                    "algorithmic_bytes_per_call": 4 * B * H * S * d + B * S, "library": pkg.version()},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                     "frac": achieved / INT8_PEAK_TOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "frac": achieved / INT8_PEAK_TOPS,
+                     "traffic": None if args.full_range_p else MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "kernel_us": kernel_ms * 1e3},
     }
 
     # parity of the very buffer the timed steps wrote, against the CPU checker on a few heads
     orc = g.load_oracle()
     nh = min(B * H, 4)
-    want = orc.fmha_i8_blockwise(c["q"], c["k"], c["v"], c["mask"], c["q_amax"], c["k_amax"], c["v_amax"], c["o_amax"],
-                                 heads=(0, nh))
-    st = fc.parity_stats(o.cpu().numpy().reshape(B * H, S, d)[:nh], want.reshape(B * H, S, d)[:nh])
+    if args.full_range_p:  # the first heads of batch entry 0, against the checker's 255-step mode
+        nh = min(H, 4)
+        want = orc.fmha_i8_blockwise_cross(c["q"][:1, :nh], c["k"][:1, :nh], c["v"][:1, :nh], c["mask"][:1],
+                                           c["q_amax"], c["k_amax"], c["v_amax"], c["o_amax"], block=128 if S % 128 == 0 else 64,
+                                           full_range_p=True)
+    else:
+        want = orc.fmha_i8_blockwise(c["q"], c["k"], c["v"], c["mask"], c["q_amax"], c["k_amax"], c["v_amax"],
+                                     c["o_amax"], heads=(0, nh))
+    st = fc.parity_stats(o.cpu().numpy().reshape(B * H, S, d)[:nh], want.reshape(-1, S, d)[:nh])
     out["parity"] = {"heads_checked": nh, "within_1_lsb": st["within1"], "exact": st["exact"], "max_abs_lsb": st["max"]}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(orc, c, args.cpu_heads, args.cpu_threads)
