@@ -28,6 +28,8 @@
 //     transcendental unit, the int32 accumulators of both GEMMs started at the bit pattern of a float (an MFMA inline
 //     constant) so that they can be read as floats without a convert, the running O only rescaled when a row maximum
 //     jumps by more than 2^kLazyLog2, and O normalised once, in the epilogue.
+//   * a second set of instantiations (FULLP) keeps P on all 255 steps of a byte - planned by the reference, README.md:15,186
+//     - by computing with P - 128 and starting the GEMM 2 accumulators at 128 times the column sums of the V tile.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 

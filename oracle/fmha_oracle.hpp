@@ -18,6 +18,9 @@
 // invariances), against an independent vectorised restatement and against fmha_fp32_cpu / the reference headers
 // within the reference's own 20 % criterion.  The reference holds no golden vectors for this path and its GPU
 // kernel cannot run here, so no bit-level vector from the reference kernel itself exists.
+// The full_range_p mode of fmha_i8_cpu_blockwise_cross (P on 255 steps) restates no reference code - the reference
+// only plans that variant (README.md:15,186) - and is pinned by the mathematics alone: the same closed forms and
+// invariances, an independent restatement, and its smaller distance to float64 attention.
 #pragma once
 #include <algorithm>
 #include <cmath>
