@@ -210,3 +210,15 @@ def test_full_range_p_at_the_benchmark_shape(pkg, orc, dev):
     narrow = pkg.fmha_infer_i8(*t, *_scales(c)).cpu().numpy()
     delta = np.abs(narrow.astype(int) - got.astype(int))
     assert delta.max() <= 2 and 0 < (delta != 0).mean() < 0.5
+
+
+@pytest.mark.gpu
+def test_full_range_p_exponent_offsets_of_the_order_of_a_hundred_thousand(pkg, orc, dev):
+    """Heavy-tailed Q, K and a forty-fold score scale: block maxima of 10^5 in base-2 units, where one unit in the last
+    place of the exponent offset is a percent of p.  The largest p of a row must quantise to at most 255: a 256 would
+    wrap to the byte 0 and drop the very key the row attends to most."""
+    c = fc.make_inputs(2, 3, 1152, 64, dist="student_t", sigma=1.0, seed=1128)
+    c = dict(c, q=fc.make_inputs(2, 3, 470, 64, seed=5128)["q"])
+    scales = (c["q_amax"] * 40.0, c["k_amax"], c["v_amax"], 1.0)
+    want = orc.fmha_i8_blockwise_cross(c["q"], c["k"], c["v"], c["mask"], *scales, full_range_p=True)
+    _gate(_gpu(pkg, dev, c, scales), want, "large offsets")
