@@ -222,3 +222,27 @@ def test_full_range_p_exponent_offsets_of_the_order_of_a_hundred_thousand(pkg, o
     scales = (c["q_amax"] * 40.0, c["k_amax"], c["v_amax"], 1.0)
     want = orc.fmha_i8_blockwise_cross(c["q"], c["k"], c["v"], c["mask"], *scales, full_range_p=True)
     _gate(_gpu(pkg, dev, c, scales), want, "large offsets")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("S,d", [(65536, 64), (16384, 128)])
+def test_full_range_p_longest_sequences_by_closed_forms(pkg, dev, S, d):
+    """The longest sequences the library takes: no CPU pass of that size finishes in seconds, so the checks are closed
+    forms.  Q == 0: attention is uniform over the unmasked keys, every P is 255 and the column sums carry half the
+    result; a one-key needle: O is the V row of that key, exactly."""
+    rng = np.random.default_rng(S + d + 1)
+    valid = S - 3 * 64 - 17
+    v = rng.integers(-127, 128, (1, 1, S, d), dtype=np.int8)
+    k = rng.integers(-20, 21, (1, 1, S, d), dtype=np.int8)
+    mask = np.zeros((1, S), np.int8)
+    mask[0, valid:] = 1
+    got = _gpu(pkg, dev, dict(q=np.zeros((1, 1, S, d), np.int8), k=k, v=v, mask=mask), (1.0, 1.0, 2.0, 1.0)).astype(np.int64)
+    y = 2.0 * v[0, 0, :valid].astype(np.float64).mean(axis=0)
+    want = np.broadcast_to(np.clip(np.rint(y), -127, 127), got.shape)
+    assert np.abs(got - want).max() <= 1 and (got == want).mean() > 0.99
+    j0 = (valid // 2) | 1
+    kn = k.copy()
+    kn[0, 0, j0] = 127
+    q = np.full((1, 1, S, d), 127, np.int8)
+    got = _gpu(pkg, dev, dict(q=q, k=kn, v=v, mask=mask), (30.0, 30.0, 1.0, 1.0)).astype(np.int64)
+    assert np.array_equal(got[0, 0], np.broadcast_to(v[0, 0, j0].astype(np.int64), (S, d)))
