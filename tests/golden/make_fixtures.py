@@ -33,8 +33,12 @@ def main():
         c = fc.make_inputs(seed=fc.MASTER_SEED, **kw)
         o = orc.fmha_i8_blockwise(c["q"], c["k"], c["v"], c["mask"], c["q_amax"], c["k_amax"], c["v_amax"],
                                   c["o_amax"])
+        # the same inputs through the checker's 255-step mode (P = rne(255 p); README.md:15,186 of the reference plans it)
+        o_full = orc.fmha_i8_blockwise_cross(c["q"], c["k"], c["v"], c["mask"], c["q_amax"], c["k_amax"], c["v_amax"],
+                                             c["o_amax"], full_range_p=True)
         np.savez_compressed(os.path.join(HERE, name + ".npz"), q=c["q"], k=c["k"], v=c["v"], mask=c["mask"],
-                            amax=np.array([c["q_amax"], c["k_amax"], c["v_amax"], c["o_amax"]], np.float32), o=o)
+                            amax=np.array([c["q_amax"], c["k_amax"], c["v_amax"], c["o_amax"]], np.float32), o=o,
+                            o_full_range_p=o_full)
         print(name, o.shape, "saturated:", float((np.abs(o) == 127).mean()))
 
 

@@ -246,3 +246,17 @@ def test_full_range_p_longest_sequences_by_closed_forms(pkg, dev, S, d):
     q = np.full((1, 1, S, d), 127, np.int8)
     got = _gpu(pkg, dev, dict(q=q, k=kn, v=v, mask=mask), (30.0, 30.0, 1.0, 1.0)).astype(np.int64)
     assert np.array_equal(got[0, 0], np.broadcast_to(v[0, 0, j0].astype(np.int64), (S, d)))
+
+
+import glob  # noqa: E402
+import os  # noqa: E402
+
+FIXTURES = sorted(glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*.npz")))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("path", FIXTURES, ids=[os.path.basename(p) for p in FIXTURES])
+def test_full_range_p_golden_fixture(pkg, dev, path):
+    f = np.load(path)  # allow_pickle stays False
+    c = dict(q=f["q"], k=f["k"], v=f["v"], mask=f["mask"])
+    _gate(_gpu(pkg, dev, c, tuple(float(x) for x in f["amax"])), f["o_full_range_p"], os.path.basename(path))

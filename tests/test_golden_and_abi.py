@@ -23,6 +23,8 @@ def test_checker_reproduces_fixture(orc, path):
     qa, ka, va, oa = (float(x) for x in f["amax"])
     got = orc.fmha_i8_blockwise(f["q"], f["k"], f["v"], f["mask"], qa, ka, va, oa)
     assert np.array_equal(got, f["o"])
+    full = orc.fmha_i8_blockwise_cross(f["q"], f["k"], f["v"], f["mask"], qa, ka, va, oa, full_range_p=True)
+    assert np.array_equal(full, f["o_full_range_p"]) and not np.array_equal(full, f["o"])
 
 
 def _declared_symbols():
