@@ -260,3 +260,21 @@ def test_full_range_p_golden_fixture(pkg, dev, path):
     f = np.load(path)  # allow_pickle stays False
     c = dict(q=f["q"], k=f["k"], v=f["v"], mask=f["mask"])
     _gate(_gpu(pkg, dev, c, tuple(float(x) for x in f["amax"])), f["o_full_range_p"], os.path.basename(path))
+
+
+@pytest.mark.gpu
+def test_full_range_p_through_the_cpp_harness(tmp_path):
+    """Host C++ calling FMHAInferI8CrossFullRangeP the way the reference's driver calls its launch function: the
+    reference's own sweep (B = H = 1, its eleven lengths, both head sizes) and the smallest benchmark configuration,
+    each checked inside the harness against the checker's 255-step mode."""
+    import json
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "bin", "test_fmha_i8")
+    assert os.path.exists(exe), "tests/bin/test_fmha_i8 is not built (python -c 'import __graft_entry__ as g; g.build()')"
+    js = str(tmp_path / "harness.json")
+    r = subprocess.run([exe, "--config", "1", "--sweep", "--full-range-p", "--iters", "20", "--warmup", "20", "--cpu-heads", "0",
+                        "--json", js], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+    print(r.stdout[-3000:])
+    assert r.returncode == 0
+    recs = [json.loads(l) for l in open(js)]
+    assert len(recs) == 23 and all(x["pass"] for x in recs)
