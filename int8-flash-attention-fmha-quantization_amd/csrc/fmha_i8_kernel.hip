@@ -33,6 +33,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+// No floating-point contraction by the compiler: every fused multiply-add in this file is written out
+// (__builtin_fmaf), so the bits of the result do not depend on which products the optimiser decides to fuse.
+#pragma clang fp contract(off)
+
 namespace fmha_i8_gfx950 {
 
 typedef int v2i __attribute__((ext_vector_type(2)));

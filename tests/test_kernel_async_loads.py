@@ -25,18 +25,50 @@ def _regs(line):
     return used
 
 
-@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
-def test_no_read_of_an_asynchronously_loaded_register_before_its_wait(tmp_path):
-    out = str(tmp_path / "kernel.s")
+def _assembly(path, *extra):
     subprocess.run(["hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-                    "-packed-fp32-ops", "-S", "--cuda-device-only", "-o", out, SRC], check=True, capture_output=True)
-    text = open(out).read()
+                    "-packed-fp32-ops", "-S", "--cuda-device-only", *extra, "-o", path, SRC], check=True,
+                   capture_output=True)
+    text = open(path).read()
     funcs = re.split(r"\n(?=_ZN14fmha_i8_gfx95018fmha_i8_fwd_kernel[^\n]*:\s)", text)[1:]
     assert len(funcs) == 64
+    return funcs
+
+
+@pytest.fixture(scope="module")
+def kernels(tmp_path_factory):
+    return _assembly(str(tmp_path_factory.mktemp("asm") / "kernel.s"))
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+def test_the_compiler_fuses_no_multiply_add_on_its_own(kernels, tmp_path):
+    """The source pins floating-point contraction off and writes out every fma it wants, so the result bits do not
+    depend on which products an optimiser fuses (hipcc's default is to fuse where it sees fit: two builds of the same
+    arithmetic once differed in one output LSB of a few elements per thousand).  Compiled with contraction switched
+    off on the command line, every kernel must come out the same instruction for instruction."""
+    def stream(f):
+        ops = []
+        for line in f.split("\n")[1:]:
+            t = line.split(";")[0].strip()
+            if t.startswith("s_endpgm"):
+                break
+            if t and not t.startswith(".") and not t.endswith(":"):
+                ops.append(re.sub(r"\.LBB\d+_\d+", "L", re.sub(r"_ZZN\w+", "SYM", t)))
+        return ops
+    pinned = _assembly(str(tmp_path / "kernel_off.s"), "-ffp-contract=off")
+    for a, b in zip(kernels, pinned):
+        assert a.split(":")[0] == b.split(":")[0]
+        assert stream(a) == stream(b), a.split(":")[0]
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+def test_no_read_of_an_asynchronously_loaded_register_before_its_wait(kernels):
+    funcs = kernels
     checked = 0
     for f in funcs:
         name = f.split(":")[0]
-        ragged = name.endswith("Lb1EEEvNS_10KernelArgsE")  # its prologue has alternative load paths: weaker check
+        # template arguments <D, BK, BIAS, FASTACC, RAGGED, FULLP>; a RAGGED prologue has alternative load paths: weaker check
+        ragged = re.search(r"ELb1ELb[01]EEEvNS_10KernelArgsE$", name) is not None
         lines = f.split("\n")
         issued = 0          # loads issued so far, in program order (they return in that order)
         pending = {}        # register -> (line of its load, ordinal of the load)
