@@ -348,6 +348,47 @@ def test_void_entry_point_streams_and_use_tcu_flag(pkg, orc, dev):
         check(o.cpu().numpy(), want, "void entry use_tcu=%s" % use_tcu)
 
 
+def test_concurrent_host_threads_on_their_own_streams(pkg, dev):
+    """The library keeps no state between calls (the reference's launch function has none either, src/fmha_i8.cu:157-173),
+    so any host thread may call it: four threads, each with its own stream, problem and buffers, two hundred calls each
+    of both entry points, all at once; every thread must end with exactly the bytes a single-threaded call gives."""
+    import threading
+    import torch
+    problems = []
+    for t in range(4):
+        c = fc.make_inputs(2, 2 + t, 256 + 64 * t, 64 if t % 2 else 128, pad="scatter", seed=90 + t)
+        c["mask"][:, 0] = 0
+        bufs = to_dev(dev, c["q"], c["k"], c["v"], c["mask"])
+        scales = (c["q_amax"], c["k_amax"], c["v_amax"], c["o_amax"])
+        want = [pkg.fmha_infer_i8(*bufs, *scales, full_range_p=full).cpu().numpy() for full in (False, True)]
+        problems.append((bufs, scales, want))
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(t):
+        try:
+            bufs, scales, want = problems[t]
+            stream = torch.cuda.Stream(device=dev)
+            outs = [torch.empty_like(bufs[0]), torch.empty_like(bufs[0])]
+            for _ in range(200):
+                for full in (False, True):
+                    pkg.fmha_infer_i8(*bufs, *scales, out=outs[full], stream=stream, full_range_p=full)
+            stream.synchronize()
+            for full in (False, True):
+                if not np.array_equal(outs[full].cpu().numpy(), want[full]):
+                    errors.append("thread %d, full_range_p=%s: output differs" % (t, full))
+        except Exception as e:  # noqa: BLE001 - reported by the main thread
+            errors.append("thread %d: %r" % (t, e))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=120)
+    assert not any(th.is_alive() for th in threads), "a worker did not finish"
+    assert not errors, errors
+
+
 def test_graph_capture_and_replay(pkg, orc, dev):
     """The call allocates nothing and never synchronises, so it can be recorded into a HIP graph: capture one launch,
     replay it several times with eager work and synchronisations in between and with new inputs written into the same
