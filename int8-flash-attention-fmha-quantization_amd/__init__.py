@@ -275,3 +275,21 @@ def fmha_infer_i8(q, k, v, padding_mask, q_amax, k_amax, v_amax, o_amax=1.0, out
     if st != FMHA_I8_OK:
         raise FMHAError(st, status_string(st))
     return out
+
+
+def fmha_infer_from_float(q, k, v, padding_mask, o_amax, out_dtype=None, stream=None, full_range_p=False):
+    """The flow of the reference's driver with every step on the GPU (test_fmha_i8.cpp:91-110 quantises Q, K and V on the
+    host by their abs-max, :204-222 launches the kernel, inc/utils.hpp:53 de-quantises O): q [B,H,Sq,d] and k, v
+    [B,H,S,d] are contiguous float32 or bfloat16 tensors on the GPU, padding_mask int8 [B,S] (nonzero = masked out),
+    o_amax the range the int8 output is scaled to (the driver takes max |O| of its float path).  Returns
+    (O as out_dtype - default: q's dtype -, int8 O, (q_amax, k_amax, v_amax)).  The three maxima are read back in one
+    copy because FMHAParamI8 is passed by value, as in the reference; nothing else leaves the device."""
+    import torch
+    st = stream if stream is not None else torch.cuda.current_stream(q.device)
+    with torch.cuda.stream(st):
+        (qi, qa), (ki, ka), (vi, va) = (quantize_tensor(t, stream=st) for t in (q, k, v))
+        amax = [float(x) for x in torch.cat((qa, ka, va)).cpu()]  # the one synchronisation of the flow
+    if min(amax) <= 0.0:
+        raise ValueError("q, k and v must each hold a nonzero value (abs-max %r)" % (amax,))
+    o_i8 = fmha_infer_i8(qi, ki, vi, padding_mask, amax[0], amax[1], amax[2], o_amax, stream=st, full_range_p=full_range_p)
+    return dequantize_tensor(o_i8, o_amax, stream=st, dtype=out_dtype or q.dtype), o_i8, tuple(amax)

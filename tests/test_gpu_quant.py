@@ -178,3 +178,31 @@ def test_bf16_nan_is_skipped_and_quantises_to_zero(pkg, dev):
     torch.cuda.synchronize()
     assert a.item() == float("inf")
     assert list(q.cpu().numpy()) == [0, 1, 0, -2, 0, 0, 1, 2, 127]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_float_in_float_out_flow_matches_the_host_flow(pkg, orc, dev, dtype_name):
+    """fmha_infer_from_float does on the GPU what the reference's driver does around its kernel (quantise by abs-max,
+    launch, de-quantise: test_fmha_i8.cpp:91-110,204-222, inc/utils.hpp:53).  Against the same flow on the host with
+    the checker: the int8 tensors it feeds the kernel are bit-identical, the int8 O passes the usual gate, and the float
+    O is that int8 O times o_amax / 127 exactly."""
+    import torch
+    dtype = getattr(torch, dtype_name)
+    c = fc.make_inputs(2, 3, 320, 64, pad="scatter", seed=55)
+    c["mask"][:, 0] = 0
+    floats = [torch.from_numpy(c[n]).to(dev).to(dtype).contiguous() for n in ("qf", "kf", "vf")]
+    host = [t.float().cpu().numpy() for t in floats]  # what the GPU really sees (bfloat16 rounds the inputs)
+    amax = [orc.abs_max(x) for x in host]
+    qi, ki, vi = (orc.quantize_i8(x, a) for x, a in zip(host, amax))
+    o_amax = 0.75
+    for full in (False, True):
+        o_f, o_i8, got_amax = pkg.fmha_infer_from_float(*floats, torch.from_numpy(c["mask"]).to(dev), o_amax, full_range_p=full)
+        torch.cuda.synchronize()
+        assert list(got_amax) == [float(a) for a in amax]
+        want = orc.fmha_i8_blockwise_cross(qi, ki, vi, c["mask"], *amax, o_amax, full_range_p=full)
+        st = fc.parity_stats(o_i8.cpu().numpy(), want)
+        assert st["within1"] >= 0.999 and st["max"] <= 2, (dtype_name, full, st)
+        assert o_f.dtype == dtype
+        expect = (o_i8.float().cpu() / 127.0 * o_amax).to(dtype)  # inc/utils.hpp:53, rounded once to the output type
+        assert torch.equal(o_f.cpu(), expect)
