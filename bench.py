@@ -4,9 +4,11 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--no-cpu-baseline] [--full-range-p]
 
 One "step" is one FMHAInferI8 call (through the C ABI of libfmha_i8.so) on one synthetic batch that is already
-resident in HBM.  The default warm-up is 2000 calls (about 60 ms): the shader clock needs some 40 ms of load to settle,
-and a call measured before that is up to 30 % slower than the steady state.  The default workload is the headline shape B=4, H=16, S=1024, d=128 (int8 Q/K/V quantised from
-N(0,1) with per-tensor amax, o_amax = 1, no padding).  Prints ONE JSON line:
+resident in HBM.  The shader clock needs some 40 ms of load to settle, and a call measured before that is up to 30 %
+slower than the steady state, so before the --warmup calls the same launch runs untimed for --preheat-ms milliseconds
+(default 100; reported as `preheat_ms` and `preheat_calls`, never counted in `steps` or `warmup`).  The default
+workload is the headline shape B=4, H=16, S=1024, d=128 (int8 Q/K/V quantised from N(0,1) with per-tensor amax,
+o_amax = 1, no padding).  Prints ONE JSON line:
 
   value              effective INT8 TOPS = 4*B*H*S^2*d / time (two GEMMs, 2 ops per MAC; softmax work not counted)
   us_per_call        mean microseconds per call over the timed steps
@@ -78,6 +80,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--full-range-p", action="store_true", help="time FMHAInferI8CrossFullRangeP (P on 255 steps) "
                     "instead of the reference's entry point; not the headline configuration")
+    ap.add_argument("--preheat-ms", type=float, default=100.0, help="untimed calls of the same launch before the "
+                    "warm-up, for this many milliseconds, so that the shader clock has settled (0 switches it off)")
+    ap.add_argument("--parity-heads", type=int, default=16, help="heads of the timed output checked against the CPU "
+                    "checker (spread over all batch entries)")
     ap.add_argument("--cpu-heads", type=int, default=64, help="heads in the CPU-baseline sample")
     ap.add_argument("--cpu-threads", type=int, default=16)
     args = ap.parse_args()
@@ -117,6 +123,14 @@ def main():
         if st != 0:
             raise pkg.FMHAError(st, pkg.status_string(st))
 
+    # Pre-heat: the same launch, untimed, in batches with a synchronisation between them, until the time is up.
+    preheat_calls, t_heat = 0, time.perf_counter()
+    while args.preheat_ms > 0 and (time.perf_counter() - t_heat) * 1e3 < args.preheat_ms:
+        for _ in range(200):
+            step()
+        torch.cuda.synchronize()
+        preheat_calls += 200
+    preheat_ms = (time.perf_counter() - t_heat) * 1e3 if preheat_calls else 0.0
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -140,6 +154,7 @@ def main():
     out = {
         "metric": "INT8 FMHA effective TOPS (4*B*H*S^2*d ops) at B4.H16.S1024.d128; us/call; % of int8 MFMA peak",
         "value": tops, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "preheat_ms": preheat_ms, "preheat_calls": preheat_calls,
         "ms_per_step": ms_per_step, "us_per_call": ms_per_step * 1e3,
         "pct_of_int8_peak": 100.0 * tops / INT8_PEAK_TOPS,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
@@ -157,17 +172,22 @@ def main():
     }
 
     # parity of the very buffer the timed steps wrote, against the CPU checker on a few heads
+    # `parity-heads` (batch, head) pairs spread evenly over batch*head, so that every batch entry is touched
     orc = g.load_oracle()
-    nh = min(B * H, 4)
-    if args.full_range_p:  # the first heads of batch entry 0, against the checker's 255-step mode
-        nh = min(H, 4)
-        want = orc.fmha_i8_blockwise_cross(c["q"][:1, :nh], c["k"][:1, :nh], c["v"][:1, :nh], c["mask"][:1],
-                                           c["q_amax"], c["k_amax"], c["v_amax"], c["o_amax"], block=128 if S % 128 == 0 else 64,
-                                           full_range_p=True)
+    nh = max(1, min(B * H, args.parity_heads))
+    picks = sorted({(i * B * H) // nh for i in range(nh)})
+    got_all = o.cpu().numpy().reshape(B * H, S, d)
+    # the picked heads as a problem of its own: one "batch entry" with one head per pick, each with its mask row
+    qg, kg, vg = (np.ascontiguousarray(c[n].reshape(B * H, 1, S, d)[picks]) for n in ("q", "k", "v"))
+    mg = np.ascontiguousarray(c["mask"][[bh // H for bh in picks]])
+    if args.full_range_p:  # against the checker's 255-step mode
+        want = orc.fmha_i8_blockwise_cross(qg, kg, vg, mg, c["q_amax"], c["k_amax"], c["v_amax"], c["o_amax"],
+                                           block=128 if S % 128 == 0 else 64, full_range_p=True)
     else:
-        want = orc.fmha_i8_blockwise(c["q"], c["k"], c["v"], c["mask"], c["q_amax"], c["k_amax"], c["v_amax"],
-                                     c["o_amax"], heads=(0, nh))
-    st = fc.parity_stats(o.cpu().numpy().reshape(B * H, S, d)[:nh], want.reshape(-1, S, d)[:nh])
+        want = orc.fmha_i8_blockwise(qg, kg, vg, mg, c["q_amax"], c["k_amax"], c["v_amax"], c["o_amax"])
+    got, want = list(got_all[picks]), list(np.asarray(want).reshape(len(picks), S, d))
+    st = fc.parity_stats(np.stack(got), np.stack(want))
+    nh = len(picks)
     out["parity"] = {"heads_checked": nh, "within_1_lsb": st["within1"], "exact": st["exact"], "max_abs_lsb": st["max"]}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(orc, c, args.cpu_heads, args.cpu_threads)

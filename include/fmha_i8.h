@@ -46,7 +46,8 @@ extern "C" {
 #define FMHA_I8_ERR_SEQ_LEN 3        /* a seq_len (queries or keys) <= 0 or > 65536 */
 #define FMHA_I8_ERR_BATCH_HEAD 4     /* batch_num or head_num <= 0, or the grid would exceed HIP limits */
 #define FMHA_I8_ERR_ALIGNMENT 5      /* q, k, v or o not 16-byte aligned */
-#define FMHA_I8_ERR_SCALE 6          /* an amax is not finite, o_amax <= 0, or q_amax * k_amax < 0 */
+#define FMHA_I8_ERR_SCALE 6          /* an amax is not finite, o_amax <= 0, q_amax * k_amax < 0, or a derived scale
+                                        (q_amax * k_amax / 127^2 / sqrt(d), v_amax / (128 * o_amax)) overflows */
 #define FMHA_I8_ERR_HIP_BASE 1000
 
 /* Replaces gpuImpl::FMHAInferI8 (inc/fmha_i8.h:7-15, src/fmha_i8.cu:157-173).
@@ -58,7 +59,10 @@ void FMHAInferI8(hipStream_t stream, FMHAParamI8 fmha_param, AttnDataDescriptor 
                  const void* k, const void* v, const void* padding_mask, void* o, bool use_tcu);
 
 /* Same operation, but reports what the reference cannot (its launch is unchecked, src/fmha_i8.cu:82-84):
- * FMHA_I8_OK, one of FMHA_I8_ERR_*, or FMHA_I8_ERR_HIP_BASE + hipError_t.  Never prints, never aborts. */
+ * FMHA_I8_OK, one of FMHA_I8_ERR_*, or FMHA_I8_ERR_HIP_BASE + hipError_t.  Never prints, never aborts.
+ * The hipError_t is the return value of this call's own kernel launch: the calling thread's "last error" is neither
+ * read nor cleared, so an earlier failure of some unrelated HIP call is not reported here and stays visible to the
+ * caller's own hipGetLastError(). */
 int FMHAInferI8Status(hipStream_t stream, FMHAParamI8 fmha_param, AttnDataDescriptor attn_desc, const void* q,
                       const void* k, const void* v, const void* padding_mask, void* o, bool use_tcu);
 

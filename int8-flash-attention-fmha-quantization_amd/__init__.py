@@ -285,11 +285,22 @@ def fmha_infer_from_float(q, k, v, padding_mask, o_amax, out_dtype=None, stream=
     (O as out_dtype - default: q's dtype -, int8 O, (q_amax, k_amax, v_amax)).  The three maxima are read back in one
     copy because FMHAParamI8 is passed by value, as in the reference; nothing else leaves the device."""
     import torch
-    st = stream if stream is not None else torch.cuda.current_stream(q.device)
+    if stream is None:
+        st = torch.cuda.current_stream(q.device)
+    elif isinstance(stream, torch.cuda.Stream):
+        st = stream
+    else:
+        # Every tensor of the flow is allocated by torch's caching allocator, which orders the reuse of a block by the
+        # stream it was allocated under; a raw handle gives it nothing to order by.
+        raise TypeError("stream must be a torch.cuda.Stream (or None for the current one), not %r" % type(stream))
+    # The whole flow runs with `st` as torch's current stream: the intermediate and output tensors are then allocated
+    # under the stream that the kernels writing them are queued on.
     with torch.cuda.stream(st):
         (qi, qa), (ki, ka), (vi, va) = (quantize_tensor(t, stream=st) for t in (q, k, v))
         amax = [float(x) for x in torch.cat((qa, ka, va)).cpu()]  # the one synchronisation of the flow
-    if min(amax) <= 0.0:
-        raise ValueError("q, k and v must each hold a nonzero value (abs-max %r)" % (amax,))
-    o_i8 = fmha_infer_i8(qi, ki, vi, padding_mask, amax[0], amax[1], amax[2], o_amax, stream=st, full_range_p=full_range_p)
-    return dequantize_tensor(o_i8, o_amax, stream=st, dtype=out_dtype or q.dtype), o_i8, tuple(amax)
+        if min(amax) <= 0.0:
+            raise ValueError("q, k and v must each hold a nonzero value (abs-max %r)" % (amax,))
+        o_i8 = fmha_infer_i8(qi, ki, vi, padding_mask, amax[0], amax[1], amax[2], o_amax, stream=st,
+                             full_range_p=full_range_p)
+        o = dequantize_tensor(o_i8, o_amax, stream=st, dtype=out_dtype or q.dtype)
+    return o, o_i8, tuple(amax)

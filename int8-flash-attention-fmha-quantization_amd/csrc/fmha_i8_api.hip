@@ -18,6 +18,16 @@ FMHACrossAttnDescriptor as_cross(const AttnDataDescriptor& a) {
   return FMHACrossAttnDescriptor{a.batch_num, a.seq_len, a.seq_len, a.head_num, a.head_dim};
 }
 
+// inc/fmha_i8.cuh:71-72: row_scale = 1/sqrt(d), scale_qk_out = q_amax*k_amax/127^2; folded with log2(e) because the
+// kernel's exponentials are base 2.
+float score_scale_log2(const FMHAParamI8& p, int head_dim) {
+  constexpr float kLog2e = 1.4426950408889634f;
+  const float row_scale = 1.0f / sqrtf((float)head_dim);
+  const float scale_qk_out = p.q_amax * p.k_amax / (127.f * 127.f);
+  return row_scale * scale_qk_out * kLog2e;
+}
+float output_scale(const FMHAParamI8& p) { return p.v_amax / (p.o_amax * 128.f); }  // inc/fmha_i8.cuh:318
+
 int check_args(const FMHAParamI8& p, const FMHACrossAttnDescriptor& a, const void* q, const void* k, const void* v,
                const void* mask, const void* o) {
   if (!q || !k || !v || !mask || !o) return FMHA_I8_ERR_NULL_POINTER;
@@ -33,29 +43,48 @@ int check_args(const FMHAParamI8& p, const FMHACrossAttnDescriptor& a, const voi
   // amax values are maxima of absolute values.  The kernel takes row maxima on the integer scores, which is only the
   // maximum of the scaled scores while the scale is not negative.
   if (p.q_amax * p.k_amax < 0.f) return FMHA_I8_ERR_SCALE;
+  // Finite amax values can still overflow in the scales the kernel works with (1e20 * 1e20, 1e30 / 1e-30); an
+  // infinite or NaN scale would turn every score or every output into NaN behind a status of "ok".
+  if (!isfinite(score_scale_log2(p, a.head_dim)) || !isfinite(output_scale(p))) return FMHA_I8_ERR_SCALE;
   return FMHA_I8_OK;
 }
 
 struct Variant {
   bool bias, fast, full_range_p;
 };
+// Every launch hands back the status of THAT launch (the return value of hipLaunchKernel), never the thread's last
+// error: an unrelated earlier failure of the caller must neither be reported as this call's nor be cleared by it.
 template <int D, int BK, bool RAGGED, bool FULLP>
-void launch_variant4(Variant var, dim3 grid, dim3 block, hipStream_t stream, const fmha_i8_gfx950::KernelArgs& args) {
+hipError_t launch_variant4(Variant var, dim3 grid, dim3 block, hipStream_t stream, const fmha_i8_gfx950::KernelArgs& args) {
   using namespace fmha_i8_gfx950;
-#define FMHA_LAUNCH(BB, FF) hipLaunchKernelGGL((fmha_i8_fwd_kernel<D, BK, BB, FF, RAGGED, FULLP>), grid, block, 0, stream, args)
-  if (var.bias) { if (var.fast) FMHA_LAUNCH(true, true); else FMHA_LAUNCH(true, false); }
-  else { if (var.fast) FMHA_LAUNCH(false, true); else FMHA_LAUNCH(false, false); }
+  KernelArgs by_value = args;
+  void* kernel_args[] = {&by_value};
+#ifdef FMHA_FEW_INSTANTIATIONS
+  // Test builds that are compiled many times over (tests/Makefile, target `variants`) carry only the instantiations
+  // the five benchmark configurations use: blocks of 128 keys, whole blocks, 128-step P, the one-fma merge.
+  if constexpr (BK != kBlockK || RAGGED || FULLP) return hipErrorInvalidDeviceFunction;
+  else {
+    if (!var.fast) return hipErrorInvalidDeviceFunction;
+    return var.bias ? hipLaunchKernel(reinterpret_cast<const void*>(&fmha_i8_fwd_kernel<D, BK, true, true, RAGGED, FULLP>), grid, block, kernel_args, 0, stream)
+                    : hipLaunchKernel(reinterpret_cast<const void*>(&fmha_i8_fwd_kernel<D, BK, false, true, RAGGED, FULLP>), grid, block, kernel_args, 0, stream);
+  }
+#else
+#define FMHA_LAUNCH(BB, FF) \
+  hipLaunchKernel(reinterpret_cast<const void*>(&fmha_i8_fwd_kernel<D, BK, BB, FF, RAGGED, FULLP>), grid, block, kernel_args, 0, stream)
+  if (var.bias) return var.fast ? FMHA_LAUNCH(true, true) : FMHA_LAUNCH(true, false);
+  return var.fast ? FMHA_LAUNCH(false, true) : FMHA_LAUNCH(false, false);
 #undef FMHA_LAUNCH
+#endif
 }
 template <int D, int BK, bool RAGGED>
-void launch_variant3(Variant var, dim3 grid, dim3 block, hipStream_t stream, const fmha_i8_gfx950::KernelArgs& args) {
-  if (var.full_range_p) launch_variant4<D, BK, RAGGED, true>(var, grid, block, stream, args);
-  else launch_variant4<D, BK, RAGGED, false>(var, grid, block, stream, args);
+hipError_t launch_variant3(Variant var, dim3 grid, dim3 block, hipStream_t stream, const fmha_i8_gfx950::KernelArgs& args) {
+  if (var.full_range_p) return launch_variant4<D, BK, RAGGED, true>(var, grid, block, stream, args);
+  return launch_variant4<D, BK, RAGGED, false>(var, grid, block, stream, args);
 }
 template <int D, int BK>
-void launch_variant(Variant var, dim3 grid, dim3 block, hipStream_t stream, const fmha_i8_gfx950::KernelArgs& args) {
-  if (args.seq_kv % BK != 0) launch_variant3<D, BK, true>(var, grid, block, stream, args);
-  else launch_variant3<D, BK, false>(var, grid, block, stream, args);
+hipError_t launch_variant(Variant var, dim3 grid, dim3 block, hipStream_t stream, const fmha_i8_gfx950::KernelArgs& args) {
+  if (args.seq_kv % BK != 0) return launch_variant3<D, BK, true>(var, grid, block, stream, args);
+  return launch_variant3<D, BK, false>(var, grid, block, stream, args);
 }
 
 int launch(hipStream_t stream, const FMHAParamI8& p, const FMHACrossAttnDescriptor& a, const void* q, const void* k,
@@ -74,15 +103,12 @@ int launch(hipStream_t stream, const FMHAParamI8& p, const FMHACrossAttnDescript
   args.head_num = a.head_num;
   args.q_blocks = (a.seq_len_q + fmha_i8_gfx950::kBlockQ - 1) / fmha_i8_gfx950::kBlockQ;
   args.total_wgs = a.batch_num * a.head_num * args.q_blocks;
-  // inc/fmha_i8.cuh:71-72: row_scale = 1/sqrt(d), scale_qk_out = q_amax*k_amax/127^2; folded with log2(e).
-  const float row_scale = 1.0f / sqrtf((float)a.head_dim);
-  const float scale_qk_out = p.q_amax * p.k_amax / (127.f * 127.f);
-  args.c2 = row_scale * scale_qk_out * kLog2e;
+  args.c2 = score_scale_log2(p, a.head_dim);
   // A masked score is replaced by -inf before it is scaled (see the kernel): the scale must not be exactly 0.  With
   // 1e-30 every exponent is below 1e-23 in magnitude and the probabilities are the same floats as with 0.
   if (args.c2 < 1e-30f) args.c2 = 1e-30f;
   args.floor2 = -1e6f * kLog2e;
-  args.out_scale = p.v_amax / (p.o_amax * 128.f);  // inc/fmha_i8.cuh:318
+  args.out_scale = output_scale(p);
   const dim3 grid((unsigned)args.total_wgs), block(fmha_i8_gfx950::kThreads);
   // The accumulators of Q.K^T can be read as floats without a convert when they start at the bit pattern of kBase;
   // the price is that the exponent offset (kBase*2^26 + S)*c2 is then rounded on a coarser float grid.  Take that path
@@ -100,14 +126,14 @@ int launch(hipStream_t stream, const FMHAParamI8& p, const FMHACrossAttnDescript
   const float lsb_bound = 0.0034f * fabsf(p.v_amax / p.o_amax) * sqrtf((float)(kv_padded / block_keys));
   const bool fast = lsb_bound < 0.1f;
   const Variant var{bias, fast, full_range_p};
+  hipError_t err;
   if (a.head_dim == 128) {
-    if (block_keys == fmha_i8_gfx950::kBlockK) launch_variant<128, fmha_i8_gfx950::kBlockK>(var, grid, block, stream, args);
-    else launch_variant<128, fmha_i8_gfx950::kBlockKSmall>(var, grid, block, stream, args);
+    if (block_keys == fmha_i8_gfx950::kBlockK) err = launch_variant<128, fmha_i8_gfx950::kBlockK>(var, grid, block, stream, args);
+    else err = launch_variant<128, fmha_i8_gfx950::kBlockKSmall>(var, grid, block, stream, args);
   } else {
-    if (block_keys == fmha_i8_gfx950::kBlockK) launch_variant<64, fmha_i8_gfx950::kBlockK>(var, grid, block, stream, args);
-    else launch_variant<64, fmha_i8_gfx950::kBlockKSmall>(var, grid, block, stream, args);
+    if (block_keys == fmha_i8_gfx950::kBlockK) err = launch_variant<64, fmha_i8_gfx950::kBlockK>(var, grid, block, stream, args);
+    else err = launch_variant<64, fmha_i8_gfx950::kBlockKSmall>(var, grid, block, stream, args);
   }
-  const hipError_t err = hipGetLastError();
   return err == hipSuccess ? FMHA_I8_OK : FMHA_I8_ERR_HIP_BASE + (int)err;
 }
 
@@ -157,7 +183,7 @@ const char* FMHAInferI8StatusString(int status) {
     case FMHA_I8_ERR_SEQ_LEN: return "seq_len must be between 1 and 65536 (queries and keys alike)";
     case FMHA_I8_ERR_BATCH_HEAD: return "batch_num and head_num must be positive (and the grid must fit)";
     case FMHA_I8_ERR_ALIGNMENT: return "q, k, v and o must be 16-byte aligned";
-    case FMHA_I8_ERR_SCALE: return "amax values must be finite, o_amax > 0 and q_amax * k_amax >= 0";
+    case FMHA_I8_ERR_SCALE: return "amax values must be finite, o_amax > 0, q_amax * k_amax >= 0, and the scales derived from them finite";
     default: break;
   }
   if (status >= FMHA_I8_ERR_HIP_BASE) return hipGetErrorString((hipError_t)(status - FMHA_I8_ERR_HIP_BASE));
@@ -173,6 +199,15 @@ int FMHAInferI8DebugOutOfBounds(void) {
   if (hipMemcpyFromSymbol(&count, HIP_SYMBOL(fmha_i8_gfx950::g_fmha_oob_count), sizeof(int)) != hipSuccess) return -1;
   if (hipMemcpyToSymbol(HIP_SYMBOL(fmha_i8_gfx950::g_fmha_oob_count), &zero, sizeof(int)) != hipSuccess) return -1;
   return count;
+}
+#endif
+
+#ifdef FMHA_TRACE_TICKS
+// Test build only: copies the first `words` time stamps of the last launch (see the kernel source) to host memory.
+int FMHAInferI8DebugReadTrace(unsigned* dst, int words) {
+  if (hipDeviceSynchronize() != hipSuccess) return -1;
+  if (words < 0 || words > fmha_i8_gfx950::kTraceWorkgroups * 8 * 64) return -1;
+  return hipMemcpyFromSymbol(dst, HIP_SYMBOL(fmha_i8_gfx950::g_fmha_trace), sizeof(unsigned) * words) == hipSuccess ? 0 : -1;
 }
 #endif
 

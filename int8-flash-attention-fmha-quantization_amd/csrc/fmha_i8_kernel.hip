@@ -82,6 +82,22 @@ __device__ __forceinline__ bool fmha_in_bounds(bool ok) {
 __device__ __forceinline__ constexpr bool fmha_in_bounds(bool) { return true; }
 #endif
 
+// Further test builds (tests/Makefile, target `variants`; never the shipped library).  They exist so that every claim
+// about where the time goes can be re-measured: each one removes or changes ONE thing and is timed and counted
+// against the shipped kernel.  The knock-outs produce garbage results on purpose.
+//   FMHA_KO_SOFTMAX      the block softmax is not computed (P, block maximum and row sum are left undefined)
+//   FMHA_KO_MFMA         GEMM 2 + merge and GEMM 1 + row maximum are not computed (with FMHA_KO_SOFTMAX: the key loop
+//                        is tile loads, waits and barriers only)
+//   FMHA_KO_LDS_READS    the MFMA operands are undefined registers instead of LDS reads
+//   FMHA_KO_TILE_LOADS   no K/V tile is fetched after the prologue
+//   FMHA_NO_SWIZZLE      K and V tiles lie in LDS as plain [key][d] rows (results unchanged, bank conflicts are not)
+//   FMHA_TRACE_TICKS     every wavefront records the shader-clock time of each barrier arrival and departure
+#ifdef FMHA_TRACE_TICKS
+// [workgroup][wavefront][64]: lane n of one register holds the n-th time stamp; written out when the wavefront ends.
+constexpr int kTraceWorkgroups = 4096;
+__device__ unsigned g_fmha_trace[kTraceWorkgroups * 8 * 64];
+#endif
+
 struct KernelArgs {
   const int8_t* q;
   const int8_t* k;
@@ -103,11 +119,19 @@ struct KernelArgs {
 // whose 16-lane groups touch keys {0,1,2,3,8,9,10,11} (+4, +16, +20) of a 32-key slab.
 template <int D>
 __device__ __forceinline__ int k_swizzle(int row) {
+#ifdef FMHA_NO_SWIZZLE
+  return 0;
+#else
   return D == 128 ? (row & 7) : ((row >> 1) & 3);
+#endif
 }
 template <int D>
 __device__ __forceinline__ int v_swizzle(int key) {
+#ifdef FMHA_NO_SWIZZLE
+  return 0;
+#else
   return D == 128 ? ((key & 3) | ((key >> 1) & 4)) : (((key >> 1) & 1) | ((key >> 2) & 2));
+#endif
 }
 
 // P packing: four floats y_i in [-1, 1] -> four int8 bytes rne(32767 * y_i).  v_cvt_pknorm_i16_f32 converts two at a
@@ -242,7 +266,11 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(dst), "v"(src), "s"(gbase) : "memory");
   };
+  bool prologue_done = false;  // (FMHA_KO_TILE_LOADS)
   auto issue_region = [&](const int8_t* gbase, int kb, int which, int goff, int it) {  // which: 0 = K, 1 = V
+#ifdef FMHA_KO_TILE_LOADS
+    if (prologue_done) return;
+#endif
     if (RAGGED && short_seq) {
       issue_short_region(gbase, which, goff, it);
       return;
@@ -275,7 +303,21 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   };
   auto wait_all = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+#ifdef FMHA_TRACE_TICKS
+  unsigned trace_reg = 0;
+  int trace_n = 0;
+  auto stamp = [&]() {
+    unsigned long long t;
+    asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t) :: "memory");
+    if (trace_n < 64)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tv_writelane_b32 %0, %1, m0" : "+v"(trace_reg) : "s"((unsigned)t), "s"(trace_n));
+    ++trace_n;
+  };
+  stamp();
+  auto barrier = [&]() { stamp(); asm volatile("s_barrier" ::: "memory"); stamp(); };
+#else
   auto barrier = [&]() { asm volatile("s_barrier" ::: "memory"); };
+#endif
 
   // Loads of the prologue, all issued before any is waited for and all by inline assembly, so that every wait is an
   // explicit s_waitcnt vmcnt(n) that counts the loads still allowed in flight (memory reads return in issue order):
@@ -415,17 +457,28 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // GEMM 1: S^T[key][query] = K . Q^T, int32 (inc/fmha_i8.cuh:120-172), one 32-key tile after the other; the row
   // maximum of tile t-1 is taken while the MFMAs of tile t run.  mx covers tiles 0 .. kKeyTiles-2 on return.
   auto phase_gemm1 = [&](int kb, v16i (&acc)[kKeyTiles], int (&mx)[2]) {
+#ifdef FMHA_KO_MFMA
+#pragma unroll
+    for (int t = 0; t < kKeyTiles; ++t) asm volatile("" : "=v"(acc[t]));
+    asm volatile("" : "=v"(mx[0]), "=v"(mx[1]));
+    return;
+#endif
     const int8_t* lds_k = &lds[kb & (kStages - 1)][0][0];
     const v16i zero_c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     v4i ka[2][kDSteps];  // operand reads run one key tile ahead of the MFMAs that consume them
+#ifdef FMHA_KO_LDS_READS
+    auto read_k = [&](int) { v4i undefined; asm volatile("" : "=v"(undefined)); return undefined; };
+#else
+    auto read_k = [&](int off) { return *reinterpret_cast<const v4i*>(lds_k + off); };
+#endif
 #pragma unroll
-    for (int kk = 0; kk < kDSteps; ++kk) ka[0][kk] = *reinterpret_cast<const v4i*>(lds_k + k_read_off[kk]);
+    for (int kk = 0; kk < kDSteps; ++kk) ka[0][kk] = read_k(k_read_off[kk]);
 #pragma unroll
     for (int t = 0; t < kKeyTiles; ++t) {
       if (t + 1 < kKeyTiles) {
 #pragma unroll
         for (int kk = 0; kk < kDSteps; ++kk)
-          ka[(t + 1) & 1][kk] = *reinterpret_cast<const v4i*>(lds_k + k_read_off[kk] + 32 * (t + 1) * D);
+          ka[(t + 1) & 1][kk] = read_k(k_read_off[kk] + 32 * (t + 1) * D);
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -445,6 +498,12 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // (sf(t,r) below: the score as a float; with BIAS that is kBase + S * 2^-26, and the exponent offset removes kBase.)
   // block softmax (inc/fmha_i8.cuh:174-253)
   auto phase_softmax = [&](int kb, int cls, v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles], int (&mx)[2]) {
+#ifdef FMHA_KO_SOFTMAX
+#pragma unroll
+    for (int t = 0; t < kKeyTiles; ++t) asm volatile("" : "=v"(pk[t]));
+    asm volatile("" : "=v"(m_blk), "=v"(l_blk));
+    return;
+#endif
     auto sf = [&](int t, int r) -> float { return BIAS ? __int_as_float(acc[t][r]) : (float)acc[t][r]; };
     l_blk = 0.f;
     if (cls != 0) {
@@ -559,6 +618,17 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   constexpr bool kLoadsInMfmaPhase = D == 64;
   static_assert(!kLoadsInMfmaPhase || 2 * kRegionsPerWave <= kDSteps, "one tile load per output tile of GEMM 2");
   auto phase_gemm2_merge = [&](int kb, const v4i (&pk)[kKeyTiles], int k_next, int v_next) {
+#ifdef FMHA_KO_MFMA
+    if (kLoadsInMfmaPhase) {
+      issue_k(k_next);
+      issue_v(v_next);
+    }
+    // (the softmax that produced these stays: an empty statement that reads them)
+#pragma unroll
+    for (int t = 0; t < kKeyTiles; ++t) asm volatile("" :: "v"(pk[t]));
+    asm volatile("" :: "v"(m_blk), "v"(l_blk));
+    return;
+#endif
     if (__ballot(m_blk > m_ref + kLazyLog2) != 0) {
       const float m_new = fmaxf(m_ref, m_blk);
       const float keep = __builtin_amdgcn_exp2f(m_ref - m_new);
@@ -600,6 +670,14 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       }
     };
     auto read_tile = [&](int u) {
+#ifdef FMHA_KO_LDS_READS
+#pragma unroll
+      for (int t = 0; t < kKeyTiles; ++t) {
+        asm volatile("" : "=v"(va[u & 1][t][0]));
+        asm volatile("" : "=v"(va[u & 1][t][1]));
+      }
+      return;
+#endif
 #pragma unroll
       for (int t = 0; t < kKeyTiles; ++t) {
         va[u & 1][t][0] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u] + 32 * t * D));
@@ -715,6 +793,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // that waits behind the other wavefront's softmax stream leaves the MFMA pipe idle, the reverse costs nothing.
   auto raise_priority = [&]() { asm volatile("s_setprio 3" ::: "memory"); };
   auto drop_priority = [&]() { asm volatile("s_setprio 0" ::: "memory"); };
+  prologue_done = true;
   barrier();                                   // barrier 0 (K(0) landed: prologue)
   if (wave < 4) {
     if (n > 0 && works(0)) phase_gemm1(0, acc, mx);
@@ -804,6 +883,10 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     }
   }
   wait_all();  // nothing may still be writing LDS when the wavefront ends (only possible when every key is masked)
+#ifdef FMHA_TRACE_TICKS
+  stamp();
+  if (blockIdx.x < kTraceWorkgroups) g_fmha_trace[(blockIdx.x * 8 + wave) * 64 + lane] = trace_reg;
+#endif
   if (!active) return;
 
   // ---- epilogue: normalise, requantise, store (inc/fmha_i8.cuh:318-332) --------------------------------------------

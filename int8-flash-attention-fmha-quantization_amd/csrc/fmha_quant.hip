@@ -3,6 +3,7 @@
 // kernels whose only cost is HBM traffic: 128-bit loads, one wavefront instruction covers 1 KiB of contiguous input,
 // a few thousand wavefronts in flight, no LDS except for the block reduction of the maximum.
 #include <hip/hip_runtime.h>
+#include <tuple>
 #include <stdint.h>
 
 #include "../../include/fmha_quant.h"
@@ -265,10 +266,17 @@ inline int quant_blocks(long long n) {
   return (int)(want < 1 ? 1 : (want > kQuantMaxBlocks ? kQuantMaxBlocks : want));
 }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
-inline int launch_status() {
-  const hipError_t err = hipGetLastError();
-  return err == hipSuccess ? FMHA_I8_OK : FMHA_I8_ERR_HIP_BASE + (int)err;
+// Launches report the status of the launch itself (what hipLaunchKernel returns), not the calling thread's last
+// error: an earlier failure that has nothing to do with this library is neither reported as ours nor cleared.
+template <typename... Params, typename... Args>
+inline hipError_t launch_kernel(void (*kernel)(Params...), int blocks, int threads, hipStream_t stream, Args... args) {
+  std::tuple<Params...> by_value{static_cast<Params>(args)...};
+  void* ptrs[sizeof...(Params)];
+  int i = 0;
+  std::apply([&](auto&... a) { ((ptrs[i++] = static_cast<void*>(&a)), ...); }, by_value);
+  return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(blocks), dim3(threads), ptrs, 0, stream);
 }
+inline int status_of(hipError_t err) { return err == hipSuccess ? FMHA_I8_OK : FMHA_I8_ERR_HIP_BASE + (int)err; }
 
 }  // namespace fmha_i8_gfx950
 
@@ -278,9 +286,9 @@ int FMHAAbsMaxF32(hipStream_t stream, const float* x, long long n, float* amax_o
   using namespace fmha_i8_gfx950;
   if (amax_out == nullptr || (x == nullptr && n > 0) || n < 0) return FMHA_I8_ERR_NULL_POINTER;
   if (!aligned16(x)) return FMHA_I8_ERR_ALIGNMENT;
-  hipLaunchKernelGGL(zero_float_kernel, dim3(1), dim3(1), 0, stream, amax_out);
-  if (n > 0) hipLaunchKernelGGL(abs_max_kernel, dim3(quant_blocks(n)), dim3(kQuantThreads), 0, stream, x, n, amax_out);
-  return launch_status();
+  hipError_t err = launch_kernel(zero_float_kernel, 1, 1, stream, amax_out);
+  if (err == hipSuccess && n > 0) err = launch_kernel(abs_max_kernel, quant_blocks(n), kQuantThreads, stream, x, n, amax_out);
+  return status_of(err);
 }
 
 int FMHAQuantizeI8(hipStream_t stream, const float* x, long long n, float amax_host, const float* amax_dev, int8_t* out) {
@@ -290,12 +298,8 @@ int FMHAQuantizeI8(hipStream_t stream, const float* x, long long n, float amax_h
   if (amax_dev == nullptr && !(amax_host == amax_host)) return FMHA_I8_ERR_SCALE;
   if (n == 0) return FMHA_I8_OK;
   if (5 * n > kCacheBytes)
-    hipLaunchKernelGGL(quantize_i8_kernel<true>, dim3(quant_blocks(n)), dim3(kQuantThreads), 0, stream, x, n, amax_host,
-                       amax_dev, out);
-  else
-    hipLaunchKernelGGL(quantize_i8_kernel<false>, dim3(quant_blocks(n)), dim3(kQuantThreads), 0, stream, x, n, amax_host,
-                       amax_dev, out);
-  return launch_status();
+    return status_of(launch_kernel(quantize_i8_kernel<true>, quant_blocks(n), kQuantThreads, stream, x, n, amax_host, amax_dev, out));
+  return status_of(launch_kernel(quantize_i8_kernel<false>, quant_blocks(n), kQuantThreads, stream, x, n, amax_host, amax_dev, out));
 }
 
 int FMHADequantizeI8(hipStream_t stream, const int8_t* x, long long n, float amax, float* out) {
@@ -304,20 +308,18 @@ int FMHADequantizeI8(hipStream_t stream, const int8_t* x, long long n, float ama
   if (!aligned16(x) || !aligned16(out)) return FMHA_I8_ERR_ALIGNMENT;
   if (n == 0) return FMHA_I8_OK;
   if (5 * n > kCacheBytes)
-    hipLaunchKernelGGL(dequantize_i8_kernel<true>, dim3(quant_blocks(n)), dim3(kQuantThreads), 0, stream, x, n, amax, out);
-  else
-    hipLaunchKernelGGL(dequantize_i8_kernel<false>, dim3(quant_blocks(n)), dim3(kQuantThreads), 0, stream, x, n, amax, out);
-  return launch_status();
+    return status_of(launch_kernel(dequantize_i8_kernel<true>, quant_blocks(n), kQuantThreads, stream, x, n, amax, out));
+  return status_of(launch_kernel(dequantize_i8_kernel<false>, quant_blocks(n), kQuantThreads, stream, x, n, amax, out));
 }
 
 int FMHAAbsMaxBF16(hipStream_t stream, const uint16_t* x, long long n, float* amax_out) {
   using namespace fmha_i8_gfx950;
   if (amax_out == nullptr || (x == nullptr && n > 0) || n < 0) return FMHA_I8_ERR_NULL_POINTER;
   if (!aligned16(x)) return FMHA_I8_ERR_ALIGNMENT;
-  hipLaunchKernelGGL(zero_float_kernel, dim3(1), dim3(1), 0, stream, amax_out);
-  if (n > 0)
-    hipLaunchKernelGGL(abs_max_bf16_kernel, dim3(quant_blocks(n / 2)), dim3(kQuantThreads), 0, stream, x, n, amax_out);
-  return launch_status();
+  hipError_t err = launch_kernel(zero_float_kernel, 1, 1, stream, amax_out);
+  if (err == hipSuccess && n > 0)
+    err = launch_kernel(abs_max_bf16_kernel, quant_blocks(n / 2), kQuantThreads, stream, x, n, amax_out);
+  return status_of(err);
 }
 
 int FMHAQuantizeI8BF16(hipStream_t stream, const uint16_t* x, long long n, float amax_host, const float* amax_dev,
@@ -328,12 +330,8 @@ int FMHAQuantizeI8BF16(hipStream_t stream, const uint16_t* x, long long n, float
   if (amax_dev == nullptr && !(amax_host == amax_host)) return FMHA_I8_ERR_SCALE;
   if (n == 0) return FMHA_I8_OK;
   if (3 * n > kCacheBytes)
-    hipLaunchKernelGGL(quantize_i8_bf16_kernel<true>, dim3(quant_blocks(n / 2)), dim3(kQuantThreads), 0, stream, x, n,
-                       amax_host, amax_dev, out);
-  else
-    hipLaunchKernelGGL(quantize_i8_bf16_kernel<false>, dim3(quant_blocks(n / 2)), dim3(kQuantThreads), 0, stream, x, n,
-                       amax_host, amax_dev, out);
-  return launch_status();
+    return status_of(launch_kernel(quantize_i8_bf16_kernel<true>, quant_blocks(n / 2), kQuantThreads, stream, x, n, amax_host, amax_dev, out));
+  return status_of(launch_kernel(quantize_i8_bf16_kernel<false>, quant_blocks(n / 2), kQuantThreads, stream, x, n, amax_host, amax_dev, out));
 }
 
 int FMHADequantizeI8BF16(hipStream_t stream, const int8_t* x, long long n, float amax, uint16_t* out) {
@@ -342,10 +340,8 @@ int FMHADequantizeI8BF16(hipStream_t stream, const int8_t* x, long long n, float
   if (!aligned16(x) || !aligned16(out)) return FMHA_I8_ERR_ALIGNMENT;
   if (n == 0) return FMHA_I8_OK;
   if (3 * n > kCacheBytes)
-    hipLaunchKernelGGL(dequantize_i8_bf16_kernel<true>, dim3(quant_blocks(n / 2)), dim3(kQuantThreads), 0, stream, x, n, amax, out);
-  else
-    hipLaunchKernelGGL(dequantize_i8_bf16_kernel<false>, dim3(quant_blocks(n / 2)), dim3(kQuantThreads), 0, stream, x, n, amax, out);
-  return launch_status();
+    return status_of(launch_kernel(dequantize_i8_bf16_kernel<true>, quant_blocks(n / 2), kQuantThreads, stream, x, n, amax, out));
+  return status_of(launch_kernel(dequantize_i8_bf16_kernel<false>, quant_blocks(n / 2), kQuantThreads, stream, x, n, amax, out));
 }
 
 }  // extern "C"

@@ -77,6 +77,12 @@ def test_argument_checks_need_no_gpu(pkg):
     assert pkg.FMHAInferI8CheckArgs(pkg.FMHAParamI8(1, 1, 1, 0.0), ok, a16, a16, a16, a16, a16) == pkg.FMHA_I8_ERR_SCALE
     assert pkg.FMHAInferI8CheckArgs(pkg.FMHAParamI8(float("nan"), 1, 1, 1), ok, a16, a16, a16, a16, a16) == \
         pkg.FMHA_I8_ERR_SCALE
+    # finite amax values whose product or quotient overflows: the derived scales would be inf / NaN
+    for bad in (pkg.FMHAParamI8(1e20, 1e20, 1, 1), pkg.FMHAParamI8(1, 1, 3e38, 1e-3), pkg.FMHAParamI8(3e38, 3e38, 1, 1)):
+        assert pkg.FMHAInferI8CheckArgs(bad, ok, a16, a16, a16, a16, a16) == pkg.FMHA_I8_ERR_SCALE
+        # the launching entry point refuses it before any HIP call (no GPU needed to see that)
+        assert pkg.FMHAInferI8Status(None, bad, ok, a16, a16, a16, a16, a16, True) == pkg.FMHA_I8_ERR_SCALE
+    assert pkg.FMHAInferI8CheckArgs(pkg.FMHAParamI8(1e18, 1e18, 1e30, 1e-5), ok, a16, a16, a16, a16, a16) == pkg.FMHA_I8_OK
     for code in range(0, 7):
         assert pkg.status_string(code)
 
