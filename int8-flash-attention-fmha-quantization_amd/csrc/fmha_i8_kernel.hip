@@ -91,6 +91,7 @@ __device__ __forceinline__ constexpr bool fmha_in_bounds(bool) { return true; }
 //   FMHA_KO_LDS_READS    the MFMA operands are undefined registers instead of LDS reads
 //   FMHA_KO_TILE_LOADS   no K/V tile is fetched after the prologue
 //   FMHA_NO_SWIZZLE      K and V tiles lie in LDS as plain [key][d] rows (results unchanged, bank conflicts are not)
+//   FMHA_OLD_K_SWIZZLE   the K swizzle this kernel had first, which leaves a two-way conflict on every K operand read
 //   FMHA_TRACE_TICKS     every wavefront records the shader-clock time of each barrier arrival and departure
 #ifdef FMHA_TRACE_TICKS
 // [workgroup][wavefront][64]: lane n of one register holds the n-th time stamp; written out when the wavefront ends.
@@ -122,7 +123,13 @@ __device__ __forceinline__ int k_swizzle(int row) {
 #ifdef FMHA_NO_SWIZZLE
   return 0;
 #else
-  return D == 128 ? (row & 7) : ((row >> 1) & 3);
+  // Sixteen lanes are served per cycle: rows r .. r+15 of one 16-byte chunk column.  A row is D bytes, the banks repeat
+  // every 256 bytes, so rows 256/D apart start in the same bank: those rows must get different chunks.
+#ifdef FMHA_OLD_K_SWIZZLE
+  return D == 128 ? (row & 7) : ((row >> 1) & 3);   // (two-way conflicts: rows r and r+8 / r+4 collide)
+#else
+  return D == 128 ? ((row >> 1) & 7) : ((row >> 2) & 3);
+#endif
 #endif
 }
 template <int D>
@@ -226,8 +233,10 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   const int ld_row_in = lane / kChunks;
   {
     const int row_in = ld_row_in, p = lane % kChunks;
-    const int vrow = (D == 128) ? (row_in | ((wave & 1) << 3)) : row_in;  // row bits the V swizzle looks at
-    ld_goff_k = row_in * D + ((p ^ k_swizzle<D>(row_in)) << 4);
+    // A 1 KiB region is 8 rows at D = 128 and this wavefront's regions all have the parity of its index: that is the
+    // one row bit beyond row_in that the swizzles look at.
+    const int vrow = (D == 128) ? (row_in | ((wave & 1) << 3)) : row_in;
+    ld_goff_k = row_in * D + ((p ^ k_swizzle<D>(vrow)) << 4);
     ld_goff_v = row_in * D + ((p ^ v_swizzle<D>(vrow)) << 4);
   }
   int k_read_off[kDSteps];  // + 32*t*D per key tile
