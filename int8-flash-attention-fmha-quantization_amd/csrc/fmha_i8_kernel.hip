@@ -902,6 +902,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // l_run sums 128 p / 32767 and O sums 128 p v, so mean(v) = O / (32767 l_run); a row with no unmasked key yields 0
   const float fin = (l_run > 0.f) ? args.out_scale * (128.f / kSnorm) * kBaseScale / l_run : 0.f;
   const float corr = FASTACC ? (FULLP ? -kBaseFull * t_run : kBase * t_run) : 0.f;
+  float magic_lo = kMagic - 127.f, magic_hi = kMagic + 127.f;
+  asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));  // register operands, like magic
   int w[kDSteps][4];  // w[u][a]: the four int8 of output dims 32u + 8a + 4g .. +3 of query row i32
 #pragma unroll
   for (int u = 0; u < kDSteps; ++u)
@@ -909,8 +911,11 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     for (int a = 0; a < 4; ++a) {
       float y[4];
 #pragma unroll
-      for (int bb = 0; bb < 4; ++bb) y[bb] = __builtin_amdgcn_fmed3f((o_f[u][4 * a + bb] + corr) * fin, -127.f, 127.f) + magic;
-      // magic + y holds rne(y) in the low mantissa byte (round-half-even)
+      // magic + y holds rne(y) in the low mantissa bits (round-half-even): one fma rounds the scaled output once, and
+      // the clamp to [-127, 127] (inc/fmha_i8.cuh:327-328) is taken on the sum, between magic - 127 and magic + 127
+      for (int bb = 0; bb < 4; ++bb)
+        y[bb] = __builtin_amdgcn_fmed3f(__builtin_fmaf(FASTACC ? o_f[u][4 * a + bb] + corr : o_f[u][4 * a + bb], fin, magic),
+                                        magic_lo, magic_hi);
       const int lo = __builtin_amdgcn_perm(__float_as_int(y[1]), __float_as_int(y[0]), 0x0c0c0400);
       const int hi = __builtin_amdgcn_perm(__float_as_int(y[3]), __float_as_int(y[2]), 0x0c0c0400);
       w[u][a] = __builtin_amdgcn_perm(hi, lo, 0x05040100);
