@@ -319,7 +319,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     unsigned long long t;
     asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t) :: "memory");
     if (trace_n < 64)
-      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tv_writelane_b32 %0, %1, m0" : "+v"(trace_reg) : "s"((unsigned)t), "s"(trace_n));
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tv_writelane_b32 %0, %1, m0" : "+v"(trace_reg) : "s"((unsigned)t), "s"(__builtin_amdgcn_readfirstlane(trace_n)));
     ++trace_n;
   };
   stamp();
@@ -759,6 +759,14 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // vector memory path takes 64 bytes per cycle and all eight wavefronts queue up).  K(i+3) and V(i+2) are issued
   // after Y(i), at the end of the softmax phase, or (d = 64) inside the MFMA phase that follows it; both stages were
   // last read in tick 2i-1.  Issue order per wavefront: K0 V0 | K1 K2 V1 | K3 V2 | K4 V3 | ...
+  // At d = 128 (not FULLP) the odd barriers are left out: they publish nothing - K(m) and V(m-1) are published by
+  // barrier 2m - and a stage is refilled a whole key block after its last read either way.  Between two barriers
+  // wavefronts 0..3 then run M(i) Y(i) and wavefronts 4..7 run Y(i-1) M(i), still in anti-phase, but without meeting
+  // in the middle: -2 % at S = 1024 and -2.5 % at S = 4096.  Wavefronts 0..3 then issue their tile loads right after
+  // the barrier, in front of their MFMA phase, like wavefronts 4..7 do in front of theirs (another -0.7 %).  At d = 64
+  // the two phases differ too much in length for this (+15 %), and FULLP needs barrier 2m+1 to publish the column sums.
+  constexpr bool kOneBarrier = D == 128 && !FULLP;
+  auto barrier_odd = [&]() { if (!kOneBarrier) barrier(); };
   const int n = kb_end;
   auto cls_of = [&](int kb) { return __builtin_amdgcn_readfirstlane((int)lds_class[kb]); };
   auto works = [&](int kb) { return active && !(cls_of(kb) & 2); };  // nothing in a fully masked block is attended to
@@ -781,8 +789,14 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // Before barrier 2m every wavefront waits for its share of K(m) and V(m-1).  The tiles issued since may stay in
   // flight: the pair of the previous issue point and, for wavefronts 0..3 when they issue after the softmax (they
   // have just done so), the pair of this one.
-  auto wait_tiles = [&](bool issued_after_softmax) { wait_all_but(!kLoadsInMfmaPhase && issued_after_softmax ? 4 : 2); };
+  auto wait_tiles = [&](bool issued_after_softmax) {
+    wait_all_but(!kLoadsInMfmaPhase && !kOneBarrier && issued_after_softmax ? 4 : 2);
+  };
   auto issue_after_softmax = [&](int i) { if (!kLoadsInMfmaPhase) issue_for(i); };
+  // wavefronts 0..3: the same pair of tiles either after the softmax or, with one barrier per key block, after the
+  // barrier that follows it
+  auto issue_after_softmax_a = [&](int i) { if (!kOneBarrier) issue_after_softmax(i); };
+  auto issue_after_barrier_a = [&](int i) { if (kOneBarrier) issue_after_softmax(i); };
   // FULLP: V(m) is summed by wavefronts 4..7 in tick 2m+1, one tick before its GEMM 2, so it is barrier 2m+1 that
   // publishes it.  Wavefronts 0..3 arrive there from their MFMA phase (the pair issued last may stay in flight),
   // wavefronts 4..7 from their softmax (the pair they have just issued; none where the loads go out in the MFMA phase).
@@ -816,11 +830,12 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       for (; i + 1 < n && i + 1 < kb_plain; ++i) {
         v4i pk[kKeyTiles];
         wait_v_for_colsum_a();
-        barrier();
+        barrier_odd();
         phase_softmax(i, 0, acc, pk, mx);
-        issue_after_softmax(i);
+        issue_after_softmax_a(i);
         wait_tiles(true);
         barrier();
+        issue_after_barrier_a(i);
         raise_priority();
         phase_gemm2_merge(i, pk, min(i + 3, last), min(i + 2, last));
         phase_gemm1(i + 1, acc, mx);
@@ -832,11 +847,12 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       const bool work = active && !(cls & 2);
       v4i pk[kKeyTiles];
       wait_v_for_colsum_a();
-      barrier();                               // barrier 2i+1
+      barrier_odd();                           // barrier 2i+1
       if (work) phase_softmax(i, cls, acc, pk, mx);
-      issue_after_softmax(i);
+      issue_after_softmax_a(i);
       wait_tiles(true);
       barrier();                               // barrier 2i+2
+      issue_after_barrier_a(i);
       raise_priority();
       if (work) phase_gemm2_merge(i, pk, min(i + 3, last), min(i + 2, last));
       else issue_in_mfma_phase(i);
@@ -844,11 +860,11 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       else forget_scores();
       drop_priority();
     }
-    barrier();                                 // barrier 2n+1: wavefronts 4..7 run their last MFMA phase after it
+    barrier_odd();                             // barrier 2n+1: wavefronts 4..7 run their last MFMA phase after it
   } else {
     issue_first();
     if (FULLP) wait_all_but(3);                // V(0) has landed: K1 K2 V1 may be in flight
-    barrier();                                 // barrier 1
+    barrier_odd();                             // barrier 1
     if (FULLP && n > 0) phase_colsum(0);
     if (n > 0 && works(0)) phase_gemm1(0, acc, mx);
     else forget_scores();
@@ -862,7 +878,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         phase_softmax(i, 0, acc, pk, mx);
         issue_after_softmax(i);
         wait_v_for_colsum_b();
-        barrier();
+        barrier_odd();
         raise_priority();
         phase_gemm2_merge(i, pk, min(i + 3, last), min(i + 2, last));
         if (FULLP) phase_colsum(i + 1);
@@ -880,7 +896,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       if (work) phase_softmax(i, cls, acc, pk, mx);
       issue_after_softmax(i);
       wait_v_for_colsum_b();
-      barrier();                               // barrier 2i+3
+      barrier_odd();                           // barrier 2i+3
       raise_priority();
       if (work) phase_gemm2_merge(i, pk, min(i + 3, last), min(i + 2, last));
       else issue_in_mfma_phase(i);
