@@ -131,10 +131,12 @@ def main():
         torch.cuda.synchronize()
         preheat_calls += 200
     preheat_ms = (time.perf_counter() - t_heat) * 1e3 if preheat_calls else 0.0
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record(stream)  # (torch creates the HIP event at its first record: not inside the timed region)
     for _ in range(args.warmup):
         step()
+    ev1.record(stream)
     torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record(stream)
     for _ in range(args.steps):
