@@ -71,6 +71,33 @@ def cpu_baseline(orc, c, sample_heads, threads):
             "seconds": dt, "us_per_call_extrapolated": dt / sample_heads * B * H * 1e6}
 
 
+def sample_clock(step, burst):
+    """Queues `burst` launches and reads /sys/class/drm/card*/device/pp_dpm_sclk (the level marked '*') and the board
+    power while they run.  Returns {} where the files do not exist or cannot be read."""
+    import glob
+    import re
+    import torch
+    for _ in range(burst):
+        step()
+    time.sleep(0.2)  # (the read-outs lag the load by tens of milliseconds)
+    got = {}
+    try:
+        for f in glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"):
+            m = re.search(r"(\d+)\s*Mhz\s*\*", open(f).read())
+            if m:
+                got["sclk_mhz_under_load"] = int(m.group(1))
+                break
+        for f in glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"):
+            got["board_power_w"] = int(open(f).read().strip()) / 1e6
+            break
+    except (OSError, ValueError):
+        pass
+    torch.cuda.synchronize()
+    if "sclk_mhz_under_load" in got:
+        got["int8_peak_tops_at_that_clock"] = 256 * 8192 * got["sclk_mhz_under_load"] * 1e6 / 1e12
+    return got
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -172,6 +199,11 @@ def main():
                      "traffic": None if args.full_range_p else MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "kernel_us": kernel_ms * 1e3},
     }
+
+    # The shader clock this box settles at under this very load (it is power-managed: boxes of one pool differ by 10 %
+    # and more): a burst of the same launch (0.3 s of work) is queued - the host is far ahead of the GPU - and the driver's clock and
+    # power read-outs are sampled while the GPU works through it.  After the timed region, so it costs it nothing.
+    out["clock"] = sample_clock(step, max(1000, int(0.3 / (kernel_ms * 1e-3))))
 
     # parity of the very buffer the timed steps wrote, against the CPU checker on a few heads
     # `parity-heads` (batch, head) pairs spread evenly over batch*head, so that every batch entry is touched
