@@ -331,6 +331,31 @@ def test_one_hot_attention_closed_form_on_gpu(pkg, dev):
 
 
 # ---- API behaviour -----------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("B,H,S,d,pad", [(4, 16, 1024, 128, "none"), (2, 4, 2048, 128, "tail256"), (1, 3, 1337, 128, "scatter"),
+                                         (2, 2, 2048, 64, "none"), (1, 2, 704, 64, "scatter")])
+def test_back_to_back_launches_write_the_same_bytes(pkg, dev, B, H, S, d, pad):
+    # The K/V tiles live in a ring of LDS stages that is refilled while other wavefronts still compute: a stage
+    # refilled too early, or read before it is published, would show as launches of one problem that differ.  200
+    # launches back to back into alternating output buffers, every one compared with the first on the GPU.
+    import torch
+    Sp = (S + 63) // 64 * 64
+    c = fc.make_inputs(B, H, Sp, d, pad="scatter" if pad == "scatter" else pad, seed=77)
+    q, k, v = (np.ascontiguousarray(c[n][:, :, :S]) for n in ("q", "k", "v"))
+    m = np.ascontiguousarray(c["mask"][:, :S])
+    m[:, 0] = 0
+    tq, tk, tv, tm = to_dev(dev, q, k, v, m)
+    outs = [torch.empty_like(tq), torch.empty_like(tq), torch.empty_like(tq)]
+    args = (c["q_amax"], c["k_amax"], c["v_amax"], c["o_amax"])
+    pkg.fmha_infer_i8(tq, tk, tv, tm, *args, out=outs[0])
+    differing = torch.zeros((), dtype=torch.int64, device=dev)
+    for it in range(200):
+        o = outs[1 + it % 2]
+        pkg.fmha_infer_i8(tq, tk, tv, tm, *args, out=o)
+        differing += (o != outs[0]).sum()
+    torch.cuda.synchronize()
+    assert int(differing.item()) == 0
+
+
 def test_void_entry_point_streams_and_use_tcu_flag(pkg, orc, dev):
     import torch
     c = fc.make_inputs(2, 2, 256, 128, seed=48, valid_lengths=[256, 100])
