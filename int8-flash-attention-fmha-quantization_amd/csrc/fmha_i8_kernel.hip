@@ -94,6 +94,9 @@ __device__ __forceinline__ constexpr bool fmha_in_bounds(bool) { return true; }
 //   FMHA_NO_SWIZZLE      K and V tiles lie in LDS as plain [key][d] rows (results unchanged, bank conflicts are not)
 //   FMHA_OLD_K_SWIZZLE   the K swizzle this kernel had first, which leaves a two-way conflict on every K operand read
 //   FMHA_TRACE_TICKS     every wavefront records the shader-clock time of each barrier arrival and departure
+//   FMHA_VGPR_STAGED_LOADS  the "before" of the direct-to-LDS tile loads: in the steady-state loop at d = 128 a K/V tile
+//                        goes HBM -> registers (global_load_dwordx4) and, one key block later, registers -> LDS
+//                        (ds_write_b128), the way a kernel without LDS-DMA has to do it; same bytes in the same places
 #ifdef FMHA_TRACE_TICKS
 // [workgroup][wavefront][64]: lane n of one register holds the n-th time stamp; written out when the wavefront ends.
 constexpr int kTraceWorkgroups = 4096;
@@ -798,6 +801,50 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // barrier that follows it
   auto issue_after_softmax_a = [&](int i) { if (!kOneBarrier) issue_after_softmax(i); };
   auto issue_after_barrier_a = [&](int i) { if (kOneBarrier) issue_after_softmax(i); };
+#ifdef FMHA_VGPR_STAGED_LOADS
+  // One pair of tiles (K(i+3), V(i+2)) on its way through this wavefront's registers: loaded at the issue point of
+  // key block i, written to LDS at the issue point of key block i+1 - still a whole key block before the barrier that
+  // publishes it.  Only where the tiles would otherwise be requested in front of the MFMA phase (d = 128).
+  constexpr bool kStaged = kOneBarrier && !kLoadsInMfmaPhase && !RAGGED;
+  v4i staged[2][kRegionsPerWave];
+  int staged_kb[2] = {0, 0};
+  bool have_staged = false;
+  auto staged_write = [&]() {
+    if (!have_staged) return;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int which = 0; which < 2; ++which)
+#pragma unroll
+      for (int it = 0; it < kRegionsPerWave; ++it) {
+        asm volatile("" : "+v"(staged[which][it]));
+        const int region = (it * kWaves + wave) % kRegions;
+        *reinterpret_cast<v4i*>(&lds[staged_kb[which] & (kStages - 1)][which][region * 1024 + 16 * lane]) = staged[which][it];
+      }
+    have_staged = false;
+  };
+  auto staged_step = [&](int i) {
+    staged_write();
+    staged_kb[0] = min(i + 3, last);
+    staged_kb[1] = min(i + 2, last);
+#pragma unroll
+    for (int which = 0; which < 2; ++which)
+#pragma unroll
+      for (int it = 0; it < kRegionsPerWave; ++it) {
+        const int8_t* gp = (which ? vg : kg) + (long)staged_kb[which] * kTileBytes;
+        const int region = (it * kWaves + wave) % kRegions;
+        const int src = (which ? ld_goff_v : ld_goff_k) + region * 1024;
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(staged[which][it]) : "v"(src), "s"(gp) : "memory");
+      }
+    have_staged = true;
+  };
+  // LDS writes are not waited for by the hand-written barrier
+  auto staged_writes_done = [&]() { if (kStaged) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
+#else
+  constexpr bool kStaged = false;
+  auto staged_write = [&]() {};
+  auto staged_step = [&](int) {};
+  auto staged_writes_done = [&]() {};
+#endif
   // FULLP: V(m) is summed by wavefronts 4..7 in tick 2m+1, one tick before its GEMM 2, so it is barrier 2m+1 that
   // publishes it.  Wavefronts 0..3 arrive there from their MFMA phase (the pair issued last may stay in flight),
   // wavefronts 4..7 from their softmax (the pair they have just issued; none where the loads go out in the MFMA phase).
@@ -834,13 +881,19 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         barrier_odd();
         phase_softmax(i, 0, acc, pk, mx);
         issue_after_softmax_a(i);
+        staged_writes_done();
         wait_tiles(true);
         barrier();
-        issue_after_barrier_a(i);
+        if (kStaged) staged_step(i);
+        else issue_after_barrier_a(i);
         raise_priority();
         phase_gemm2_merge(i, pk, min(i + 3, last), min(i + 2, last));
         phase_gemm1(i + 1, acc, mx);
         drop_priority();
+      }
+      if (kStaged) {
+        staged_write();
+        staged_writes_done();
       }
     }
     for (; i < n; ++i) {
@@ -877,7 +930,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         wait_tiles(false);
         barrier();
         phase_softmax(i, 0, acc, pk, mx);
-        issue_after_softmax(i);
+        if (kStaged) staged_step(i);
+        else issue_after_softmax(i);
         wait_v_for_colsum_b();
         barrier_odd();
         raise_priority();
@@ -886,6 +940,11 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         phase_gemm1(i + 1, acc, mx);
         if (FULLP) colsum_written();
         drop_priority();
+        staged_writes_done();
+      }
+      if (kStaged) {
+        staged_write();
+        staged_writes_done();
       }
     }
     for (; i < n; ++i) {
