@@ -16,13 +16,13 @@
 //     the row (the swizzle is applied to the global address each lane fetches), so that the 128-bit operand reads of
 //     K and the transposing reads of V (ds_read_b64_tr_b8) are bank-conflict free; Q goes once per workgroup straight
 //     into MFMA operand registers;
-//   * the kernel is bound by the instruction issue of the SIMD (a VALU instruction takes 4.3 to 5.2 cycles of it, an
+//   * the kernel is bound by the instruction issue of the SIMD (a VALU instruction takes 4.3 to 4.7 cycles of it, an
 //     exponential 8.5, an MFMA 10 to 12; two wavefronts rarely issue together), so the two wavefronts that share a SIMD
 //     run in ANTI-PHASE: every key block is an MFMA phase - GEMM 2 and merge of the previous block, then GEMM 1 of this
 //     one, with the merge and the row maximum issued in the shadow of the MFMAs - and a VALU phase, the softmax;
 //     wavefronts 4..7 run one phase behind wavefronts 0..3, and the wavefront in its MFMA phase runs at raised priority,
-//     so that the MFMA pipe never waits for an issue slot.  One workgroup barrier per key block publishes the tiles; at
-//     d = 64 and with FULLP a second one separates the two phases;
+//     so that the MFMA pipe never waits for an issue slot.  One workgroup barrier per key block publishes the tiles; with
+//     FULLP a second one separates the two phases;
 //   * the softmax is written for instruction count and issue order: exp in the base-2 domain with every scale folded
 //     into one fma, v_max3 on the raw accumulators for the row maximum, P converted two at a time by
 //     v_cvt_pknorm_i16_f32 and packed by v_perm_b32, every exponential followed by instructions that do not need the

@@ -5,7 +5,8 @@
 // instruction each (eight independent register chains, inline assembly so that nothing is rescheduled): wavefront
 // group 0 (wavefronts 0..3 of a 512-thread workgroup, one per SIMD) runs stream X, group 1 stream Y, a third group an
 // MFMA stream.  Output: cycles at 2.4 GHz per instruction PAIR (one instruction of X and one of Y); about 4.3 means
-// the two issue together, about 8.5 means one after the other.
+// the two issue together, about 8.5 means one after the other.  It also measures what instruction ALIGNMENT costs: a
+// 64-bit-encoded VALU instruction at an address that is 4 mod 8 takes 5.4 to 5.7 cycles instead of 4.7.
 //
 //     tests/bin/issue_model
 #include <hip/hip_runtime.h>
@@ -44,28 +45,36 @@
 #define MF4 MF_(0) MF_(16) MF_(0) MF_(16)
 #define MF32 MF4 MF4 MF4 MF4 MF4 MF4 MF4 MF4
 
-enum Op { kNone, kAdd, kAddS, kMul, kFma, kFmaS, kFmac, kMov, kMax3, kMaxF, kPknorm, kPerm, kCvt, kExp, kMfma };
+enum Op { kNone, kAdd, kAddS, kMul, kFma, kFmaS, kFmac, kMov, kMax3, kMaxF, kPknorm, kPerm, kCvt, kExp, kMfma, kFmaMis, kPknormMis, kAddMis, kMfmaMis };
 #define CLOBBER "memory", "s20", "s21", "v0", "v1", "v2", "v3", "v4", "v5", "v6", "v7", "v8", "v9", "v10", "v11", "v12", "v13", \
     "v14", "v15", "v16", "v17", "v18", "v19", "v20", "v21", "v22", "v23", "v24", "v25", "v26", "v27", "v28", "v29", "v30",     \
     "v31", "v64", "v65", "v66", "v67", "v68", "v69", "v70", "v71", "v100", "v101", "v102", "v104", "v105", "v106", "v107",   \
     "v108", "v109", "v110", "v111"
 
+// Every stream starts at an 8-byte-aligned address (the compiler aligns nothing inside a function); the "at 4 mod 8"
+// variants start one dword later, so that every 64-bit-encoded instruction of the stream straddles an aligned pair.
+#define AL ".p2align 3\n\t"
+#define MIS ".p2align 3\n\ts_nop 0\n\t"
 template <int OP>
 __device__ __forceinline__ void stream() {
-  if (OP == kAdd) asm volatile(R192(OP_ADD) ::: CLOBBER);
-  if (OP == kAddS) asm volatile(R192(OP_ADD_S) ::: CLOBBER);
-  if (OP == kMul) asm volatile(R192(OP_MUL) ::: CLOBBER);
-  if (OP == kFma) asm volatile(R192(OP_FMA) ::: CLOBBER);
-  if (OP == kFmaS) asm volatile(R192(OP_FMA_S) ::: CLOBBER);
-  if (OP == kFmac) asm volatile(R192(OP_FMAC) ::: CLOBBER);
-  if (OP == kMov) asm volatile(R192(OP_MOV) ::: CLOBBER);
-  if (OP == kMax3) asm volatile(R192(OP_MAX3) ::: CLOBBER);
-  if (OP == kMaxF) asm volatile(R192(OP_MAXF) ::: CLOBBER);
-  if (OP == kPknorm) asm volatile(R192(OP_PKNORM) ::: CLOBBER);
-  if (OP == kPerm) asm volatile(R192(OP_PERM) ::: CLOBBER);
-  if (OP == kCvt) asm volatile(R192(OP_CVT) ::: CLOBBER);
-  if (OP == kExp) asm volatile(R192(OP_EXP) ::: CLOBBER);
-  if (OP == kMfma) asm volatile(MF32 ::: CLOBBER);
+  if (OP == kFmaMis) asm volatile(MIS R192(OP_FMA) ::: CLOBBER);
+  if (OP == kPknormMis) asm volatile(MIS R192(OP_PKNORM) ::: CLOBBER);
+  if (OP == kAddMis) asm volatile(MIS R192(OP_ADD) ::: CLOBBER);
+  if (OP == kMfmaMis) asm volatile(MIS MF32 ::: CLOBBER);
+  if (OP == kAdd) asm volatile(AL R192(OP_ADD) ::: CLOBBER);
+  if (OP == kAddS) asm volatile(AL R192(OP_ADD_S) ::: CLOBBER);
+  if (OP == kMul) asm volatile(AL R192(OP_MUL) ::: CLOBBER);
+  if (OP == kFma) asm volatile(AL R192(OP_FMA) ::: CLOBBER);
+  if (OP == kFmaS) asm volatile(AL R192(OP_FMA_S) ::: CLOBBER);
+  if (OP == kFmac) asm volatile(AL R192(OP_FMAC) ::: CLOBBER);
+  if (OP == kMov) asm volatile(AL R192(OP_MOV) ::: CLOBBER);
+  if (OP == kMax3) asm volatile(AL R192(OP_MAX3) ::: CLOBBER);
+  if (OP == kMaxF) asm volatile(AL R192(OP_MAXF) ::: CLOBBER);
+  if (OP == kPknorm) asm volatile(AL R192(OP_PKNORM) ::: CLOBBER);
+  if (OP == kPerm) asm volatile(AL R192(OP_PERM) ::: CLOBBER);
+  if (OP == kCvt) asm volatile(AL R192(OP_CVT) ::: CLOBBER);
+  if (OP == kExp) asm volatile(AL R192(OP_EXP) ::: CLOBBER);
+  if (OP == kMfma) asm volatile(AL MF32 ::: CLOBBER);
 }
 
 // wavefront group g (256 threads each: one wavefront per SIMD) runs stream X (g = 0), Y (g = 1), Z (g = 2)
@@ -117,6 +126,12 @@ int main(int argc, char** argv) {
   ROW(kFma, kNone, kNone, "v_fma_f32 alone");
   ROW(kMax3, kNone, kNone, "v_max3_i32 alone");
   ROW(kExp, kNone, kNone, "v_exp_f32 alone");
+  printf("# -- the same from an address that is 4 mod 8: a 64-bit encoding then straddles two aligned dword pairs\n");
+  ROW(kAddMis, kNone, kNone, "v_add_f32 (32-bit encoding) alone, at 4 mod 8");
+  ROW(kFmaMis, kNone, kNone, "v_fma_f32 (64-bit encoding) alone, at 4 mod 8");
+  ROW(kPknormMis, kNone, kNone, "v_cvt_pknorm_i16_f32 (64-bit) alone, at 4 mod 8");
+  ROW(kFmaMis, kFmaMis, kNone, "v_fma_f32 | v_fma_f32, both at 4 mod 8");
+  ROW(kMfmaMis, kNone, kNone, "v_mfma_i32_32x32x32_i8 alone, at 4 mod 8 (x 6)");
   printf("# -- two wavefronts per SIMD, plain fp32 arithmetic in both: they issue together\n");
   ROW(kAdd, kAdd, kNone, "v_add_f32 | v_add_f32");
   ROW(kMul, kAdd, kNone, "v_mul_f32 | v_add_f32");
