@@ -697,11 +697,16 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // (inc/fmha_i8.cuh:298-315) four elements behind each MFMA of tile u.  Normalisation is deferred to the epilogue:
   // O and l are kept relative to 2^m_ref, and m_ref only moves when some row's block maximum exceeds it by
   // 2^kLazyLog2.
-  // Where the tile loads of a block are issued: at the end of the softmax phase, or one per output tile inside GEMM 2.
-  // The loads and their address arithmetic stand in the issue stream of whichever wavefront carries them, and the
-  // barrier waits for the longer stream: at d = 64 that is the softmax wavefront (the MFMA phase is short: -7 % with
-  // the loads moved there), at d = 128 the two are level and the loads stay where the wavefront used to arrive early.
+  // Where the tile loads of a block are issued: one per output tile inside GEMM 2.  The loads and their address
+  // arithmetic stand in the issue stream of whichever wavefront carries them; inside the MFMA phase they fall into the
+  // waits of the MFMA chain (-7 % at d = 64 against issuing them after the softmax, -0.6 % at d = 128 against issuing them
+  // in front of the MFMA phase).  The other placements are kept for the test build that stages the tiles through
+  // registers, which needs the loads of a key block in one place.
+#ifdef FMHA_VGPR_STAGED_LOADS
   constexpr bool kLoadsInMfmaPhase = D == 64;
+#else
+  constexpr bool kLoadsInMfmaPhase = true;
+#endif
   static_assert(!kLoadsInMfmaPhase || 2 * kRegionsPerWave <= kDSteps, "one tile load per output tile of GEMM 2");
   auto phase_gemm2_merge = [&](int kb, const v4i (&pk)[kKeyTiles], int k_next, int v_next) {
 #ifdef FMHA_KO_MFMA
