@@ -98,7 +98,8 @@ __device__ __forceinline__ constexpr bool fmha_in_bounds(bool) { return true; }
 //                        goes HBM -> registers (global_load_dwordx4) and, one key block later, registers -> LDS
 //                        (ds_write_b128), the way a kernel without LDS-DMA has to do it; same bytes in the same places
 #ifdef FMHA_TRACE_TICKS
-// [workgroup][wavefront][64]: lane n of one register holds the n-th time stamp; written out when the wavefront ends.
+// [workgroup][wavefront][64]: lane n < 62 of one register holds the n-th time stamp (s_memtime, shader clock), lanes 62
+// and 63 the 100 MHz counter at the start and the end of the wavefront; written out when the wavefront ends.
 constexpr int kTraceWorkgroups = 4096;
 __device__ unsigned g_fmha_trace[kTraceWorkgroups * 8 * 64];
 #endif
@@ -328,11 +329,19 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   auto stamp = [&]() {
     unsigned long long t;
     asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t) :: "memory");
-    if (trace_n < 64)
+    if (trace_n < 62)
       asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tv_writelane_b32 %0, %1, m0" : "+v"(trace_reg) : "s"((unsigned)t), "s"(__builtin_amdgcn_readfirstlane(trace_n)));
     ++trace_n;
   };
   stamp();
+  // lanes 62 and 63: the constant-rate counter (100 MHz) when the wavefront starts and ends; with the first and the last
+  // s_memtime stamp it gives the shader clock the kernel actually ran at
+  auto stamp_real = [&](int slot) {
+    unsigned long long t;
+    asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t) :: "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tv_writelane_b32 %0, %1, m0" : "+v"(trace_reg) : "s"((unsigned)t), "s"(slot));
+  };
+  stamp_real(62);
   auto barrier = [&]() { stamp(); asm volatile("s_barrier" ::: "memory"); stamp(); };
 #else
   auto barrier = [&]() { asm volatile("s_barrier" ::: "memory"); };
@@ -1058,6 +1067,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   wait_all();  // nothing may still be writing LDS when the wavefront ends (only possible when every key is masked)
 #ifdef FMHA_TRACE_TICKS
   stamp();
+  stamp_real(63);
   if (blockIdx.x < kTraceWorkgroups) g_fmha_trace[(blockIdx.x * 8 + wave) * 64 + lane] = trace_reg;
 #endif
   if (!active) return;

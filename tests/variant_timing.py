@@ -90,10 +90,14 @@ def main():
         assert lib.FMHAInferI8DebugReadTrace(buf, nwg * 8 * 64) == 0
         t = np.frombuffer(buf, dtype=np.uint32).reshape(nwg, 8, 64).astype(np.int64)
         work, wait = [[], []], [[], []]
+        cycles = ticks = 0
         for wg in range(nwg):
             for w in range(8):
-                x = t[wg, w]
-                n = int(np.argmax(x == 0)) if (x == 0).any() else 64
+                x = t[wg, w, :62]
+                n = int(np.argmax(x == 0)) if (x == 0).any() else 62
+                if n >= 2 and n < 62:  # (a full stamp register has lost its last stamp)
+                    cycles += int((x[n - 1] - x[0]) & 0xffffffff)
+                    ticks += int((t[wg, w, 63] - t[wg, w, 62]) & 0xffffffff)
                 dx = np.diff(x[:n]) & 0xffffffff  # start | (arrive, leave)* | end
                 if len(dx) > 12:
                     wait[w // 4].append(dx[1::2][3:-3])
@@ -105,6 +109,9 @@ def main():
                 "work_even_ticks_mean": round(float(np.concatenate([a[0::2] for a in work[grp]]).mean()), 1),
                 "work_odd_ticks_mean": round(float(np.concatenate([a[1::2] for a in work[grp]]).mean()), 1)}
         out["tick_unit"] = "s_memtime counts, steady-state ticks only (first and last three dropped)"
+        if ticks:
+            out["shader_mhz_inside_the_kernel"] = round(100.0 * cycles / ticks, 1)  # s_memtime counts per 10 ns
+            out["wavefront_lifetime_cycles_mean"] = round(cycles / (nwg * 8.0), 1)
     print(json.dumps(out))
 
 
