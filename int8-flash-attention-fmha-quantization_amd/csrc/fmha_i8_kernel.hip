@@ -692,9 +692,9 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   };
   // The results of a split softmax are pinned where the source has them - before the barrier - and the packing behind
   // the raised priority: left alone, the compiler moves both (none of them touches memory).
-  // Where the split pays: at d = 64 (-6 %, and it makes one barrier per key block the faster choice there); at
-  // d = 128 the pipelined form, whose packing the compiler places at the head of the MFMA phase by itself, is 1 % faster.
-  constexpr bool kSplitSoftmax = D == 64;
+  // The steady-state loop uses the split form: -6 % at d = 64 (where it also makes one barrier per key block the faster
+  // choice), -2 % at d = 128 and S = 4096 against the pipelined form, whose packing the compiler places by itself.
+  constexpr bool kSplitSoftmax = true;
   auto pin_scores = [&](v16i (&acc)[kKeyTiles]) {
 #pragma unroll
     for (int t = 0; t < kKeyTiles; ++t) asm volatile("" : "+v"(acc[t]));
