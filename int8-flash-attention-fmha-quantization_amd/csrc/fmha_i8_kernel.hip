@@ -21,8 +21,7 @@
 //     run in ANTI-PHASE: every key block is an MFMA phase - GEMM 2 and merge of the previous block, then GEMM 1 of this
 //     one, with the merge and the row maximum issued in the shadow of the MFMAs - and a VALU phase, the softmax;
 //     wavefronts 4..7 run one phase behind wavefronts 0..3, and the wavefront in its MFMA phase runs at raised priority,
-//     so that the MFMA pipe never waits for an issue slot.  One workgroup barrier per key block publishes the tiles; with
-//     FULLP a second one separates the two phases;
+//     so that the MFMA pipe never waits for an issue slot.  One workgroup barrier per key block publishes the tiles;
 //   * the softmax is written for instruction count and issue order: exp in the base-2 domain with every scale folded
 //     into one fma, v_max3 on the raw accumulators for the row maximum, P converted two at a time by
 //     v_cvt_pknorm_i16_f32 and packed by v_perm_b32, every exponential followed by instructions that do not need the
@@ -97,6 +96,8 @@ __device__ __forceinline__ constexpr bool fmha_in_bounds(bool) { return true; }
 //   FMHA_VGPR_STAGED_LOADS  the "before" of the direct-to-LDS tile loads: in the steady-state loop at d = 128 a K/V tile
 //                        goes HBM -> registers (global_load_dwordx4) and, one key block later, registers -> LDS
 //                        (ds_write_b128), the way a kernel without LDS-DMA has to do it; same bytes in the same places
+//   FMHA_TWO_BARRIERS    the "before" of the one-barrier schedule: a second workgroup barrier per key block, between the
+//                        two phases (results unchanged)
 #ifdef FMHA_TRACE_TICKS
 // [workgroup][wavefront][64]: lane n < 62 of one register holds the n-th time stamp (s_memtime, shader clock), lanes 62
 // and 63 the 100 MHz counter at the start and the end of the wavefront; written out when the wavefront ends.
@@ -347,6 +348,15 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   auto barrier = [&]() { asm volatile("s_barrier" ::: "memory"); };
 #endif
 
+  // One workgroup barrier per key block, or (a test build) two: see the tick schedule below.
+  // (FULLP at d = 64 keeps two: with one it measures 10 % slower, at d = 128 4 to 7 % faster.)
+#ifdef FMHA_TWO_BARRIERS
+  constexpr bool kOneBarrier = false;
+#else
+  constexpr bool kOneBarrier = !(FULLP && D == 64);
+#endif
+  constexpr int kVAhead = (FULLP && kOneBarrier) ? 3 : 2;
+
   // Loads of the prologue, all issued before any is waited for and all by inline assembly, so that every wait is an
   // explicit s_waitcnt vmcnt(n) that counts the loads still allowed in flight (memory reads return in issue order):
   //   mask bytes of the first 2048 keys (1 load) | K0 | Q (kDSteps loads) | V0
@@ -456,7 +466,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 
   // K0 and Q have landed once at most V0 is still in flight.  The registers are redefined after the wait so that no
   // use of them can be scheduled above it.
-  asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kRegionsPerWave) : "memory");
+  // (FULLP: V0 as well - wavefronts 4..7 sum its columns right after the first barrier.)
+  asm volatile("s_waitcnt vmcnt(%0)" :: "n"(FULLP && kOneBarrier ? 0 : kRegionsPerWave) : "memory");
 #pragma unroll
   for (int kk = 0; kk < kDSteps; ++kk) asm volatile("" : "+v"(qreg[kk]));
 
@@ -854,9 +865,13 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // 2m - and a stage is refilled a whole key block after its last read either way.  Between two barriers wavefronts
   // 0..3 then run M(i) Y(i) and wavefronts 4..7 run Y(i-1) M(i), still in anti-phase, but without meeting in the
   // middle.  Where the tile loads are not issued inside the MFMA phase (d = 128), wavefronts 0..3 issue theirs right
-  // after the barrier, in front of their MFMA phase, like wavefronts 4..7 do in front of theirs.  FULLP needs barrier
-  // 2m+1 to publish the column sums.
-  constexpr bool kOneBarrier = !FULLP;
+  // after the barrier, in front of their MFMA phase, like wavefronts 4..7 do in front of theirs.
+  // FULLP: wavefronts 4..7 sum the columns of V(i+1) inside M(i), before their GEMM 1 of that block, and the sums are
+  // read in M(i+1) by everyone, behind barrier 2i+4.  V therefore runs one key block further ahead than K needs (the
+  // four V stages hold V(i) .. V(i+3)): barrier 2m publishes K(m) and V(m) instead of K(m) and V(m-1), and the first
+  // barrier V(0).  Issue order per wavefront: K0 V0 | K1 V1 K2 V2 | K3 V3 | K4 V4 | ...
+  // (FMHA_TWO_BARRIERS, a test build: the schedule with a barrier between the phases as well, in which barrier 2m+1
+  // publishes the column sums and V runs no further ahead than without FULLP.)
   auto barrier_odd = [&]() { if (!kOneBarrier) barrier(); };
   const int n = kb_end;
   auto cls_of = [&](int kb) { return __builtin_amdgcn_readfirstlane((int)lds_class[kb]); };
@@ -868,14 +883,21 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   const int last = n - 1;
   auto issue_first = [&]() {          // after barrier 0
     if (n > 0) {
-      issue_k(min(1, last));
-      issue_k(min(2, last));
-      issue_v(min(1, last));
+      if (FULLP && kOneBarrier) {  // in pairs, so that "all but the newest two tiles" means the same at every barrier
+        issue_k(min(1, last));
+        issue_v(min(1, last));
+        issue_k(min(2, last));
+        issue_v(min(2, last));
+      } else {
+        issue_k(min(1, last));
+        issue_k(min(2, last));
+        issue_v(min(1, last));
+      }
     }
   };
   auto issue_for = [&](int i) {  // where GEMM 2 of block i is skipped
     issue_k(min(i + 3, last));
-    issue_v(min(i + 2, last));
+    issue_v(min(i + kVAhead, last));
   };
   // Before barrier 2m every wavefront waits for its share of K(m) and V(m-1).  The tiles issued since may stay in
   // flight: the pair of the previous issue point and, for wavefronts 0..3 when they issue after the softmax (they
@@ -932,11 +954,11 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   auto staged_step = [&](int) {};
   auto staged_writes_done = [&]() {};
 #endif
-  // FULLP: V(m) is summed by wavefronts 4..7 in tick 2m+1, one tick before its GEMM 2, so it is barrier 2m+1 that
-  // publishes it.  Wavefronts 0..3 arrive there from their MFMA phase (the pair issued last may stay in flight),
+  // FULLP with two barriers per key block: V(m) is summed by wavefronts 4..7 in tick 2m+1, one tick before its GEMM 2,
+  // so it is barrier 2m+1 that publishes it.  Wavefronts 0..3 arrive there from their MFMA phase (the pair issued last may stay in flight),
   // wavefronts 4..7 from their softmax (the pair they have just issued; none where the loads go out in the MFMA phase).
-  auto wait_v_for_colsum_a = [&]() { if (FULLP) wait_all_but(2); };
-  auto wait_v_for_colsum_b = [&]() { if (FULLP) wait_all_but(kLoadsInMfmaPhase ? 0 : 2); };
+  auto wait_v_for_colsum_a = [&]() { if (FULLP && !kOneBarrier) wait_all_but(2); };
+  auto wait_v_for_colsum_b = [&]() { if (FULLP && !kOneBarrier) wait_all_but(kLoadsInMfmaPhase ? 0 : 2); };
   auto issue_in_mfma_phase = [&](int i) { if (kLoadsInMfmaPhase) issue_for(i); };
   v16i acc[kKeyTiles];  // S^T of the block whose softmax comes next (GEMM 1 -> softmax, across a barrier)
   int mx[2];
@@ -979,7 +1001,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
           pin_scores(acc);
           phase_pack(acc, pk);
         }
-        phase_gemm2_merge(i, pk, min(i + 3, last), min(i + 2, last));
+        phase_gemm2_merge(i, pk, min(i + 3, last), min(i + kVAhead, last));
         phase_gemm1(i + 1, acc, mx);
         drop_priority();
       }
@@ -1000,7 +1022,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       barrier();                               // barrier 2i+2
       issue_after_barrier_a(i);
       raise_priority();
-      if (work) phase_gemm2_merge(i, pk, min(i + 3, last), min(i + 2, last));
+      if (work) phase_gemm2_merge(i, pk, min(i + 3, last), min(i + kVAhead, last));
       else issue_in_mfma_phase(i);
       if (i + 1 < n && works(i + 1)) phase_gemm1(i + 1, acc, mx);
       else forget_scores();
@@ -1009,7 +1031,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     barrier_odd();                             // barrier 2n+1: wavefronts 4..7 run their last MFMA phase after it
   } else {
     issue_first();
-    if (FULLP) wait_all_but(3);                // V(0) has landed: K1 K2 V1 may be in flight
+    if (FULLP && !kOneBarrier) wait_all_but(3);  // V(0) has landed: K1 K2 V1 may be in flight
     barrier_odd();                             // barrier 1
     if (FULLP && n > 0) phase_colsum(0);
     if (n > 0 && works(0)) phase_gemm1(0, acc, mx);
@@ -1032,7 +1054,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
           pin_scores(acc);
           phase_pack(acc, pk);
         }
-        phase_gemm2_merge(i, pk, min(i + 3, last), min(i + 2, last));
+        phase_gemm2_merge(i, pk, min(i + 3, last), min(i + kVAhead, last));
         if (FULLP) phase_colsum(i + 1);
         phase_gemm1(i + 1, acc, mx);
         if (FULLP) colsum_written();
@@ -1055,7 +1077,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       wait_v_for_colsum_b();
       barrier_odd();                           // barrier 2i+3
       raise_priority();
-      if (work) phase_gemm2_merge(i, pk, min(i + 3, last), min(i + 2, last));
+      if (work) phase_gemm2_merge(i, pk, min(i + 3, last), min(i + kVAhead, last));
       else issue_in_mfma_phase(i);
       if (FULLP && i + 1 < n) phase_colsum(i + 1);
       if (i + 1 < n && works(i + 1)) phase_gemm1(i + 1, acc, mx);
