@@ -24,8 +24,10 @@
 //     so that the MFMA pipe never waits for an issue slot.  One workgroup barrier per key block publishes the tiles;
 //   * the softmax is written for instruction count and issue order: exp in the base-2 domain with every scale folded
 //     into one fma, v_max3 on the raw accumulators for the row maximum, P converted two at a time by
-//     v_cvt_pknorm_i16_f32 and packed by v_perm_b32, every exponential followed by instructions that do not need the
-//     transcendental unit, the int32 accumulators of both GEMMs started at the bit pattern of a float (an MFMA inline
+//     v_cvt_pknorm_i16_f32 and packed by v_perm_b32, the steady-state loop (blocks without masked keys) running the
+//     scale fmas, the exponentials and the sums as three dense runs with the P packing at the head of the MFMA phase,
+//     the general loop with every exponential followed by instructions that do not need the transcendental unit, the
+//     int32 accumulators of both GEMMs started at the bit pattern of a float (an MFMA inline
 //     constant) so that they can be read as floats without a convert, the running O only rescaled when a row maximum
 //     jumps by more than 2^kLazyLog2, and O normalised once, in the epilogue.
 //   * a second set of instantiations (FULLP) keeps P on all 255 steps of a byte - planned by the reference, README.md:15,186
@@ -348,7 +350,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   auto barrier = [&]() { asm volatile("s_barrier" ::: "memory"); };
 #endif
 
-  // One workgroup barrier per key block, or (a test build) two: see the tick schedule below.
+  // One workgroup barrier per key block, or (a test build) two: see the schedule below.
   // (FULLP at d = 64 keeps two: with one it measures 10 % slower, at d = 128 4 to 7 % faster.)
 #ifdef FMHA_TWO_BARRIERS
   constexpr bool kOneBarrier = false;
@@ -849,29 +851,28 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // An LDS write is not waited for by the hand-written barrier: wavefronts 4..7 do so at the end of the phase.
   auto colsum_written = [&]() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
 
-  // ---- the tick schedule -------------------------------------------------------------------------------------------
-  // A tick is the interval between two workgroup barriers.  Every key block i is two phases per wavefront: an MFMA
-  // phase M(i) = [GEMM 2 + merge of block i-1][GEMM 1 of block i] and a VALU phase Y(i) = softmax of block i.
-  // Wavefronts 0..3 run M(i) in tick 2i and Y(i) in tick 2i+1; wavefronts 4..7 run one tick behind, so the MFMA phase
-  // of one always overlaps the VALU phase of the other wavefront of the same SIMD.  The two share one issue port: a
-  // tick lasts about as long as the issue time of both phases together, and the barrier waits for the wavefront whose
-  // own instruction stream - vector, scalar and memory instructions alike - is the longer one.
-  // Tiles: K(j), V(j) live in stage j mod 4; K(j) is read in ticks 2j and 2j+1, V(j) in ticks 2j+2 and 2j+3, and
-  // barrier 2m publishes K(m) and V(m-1).  A wavefront is held for hundreds of cycles when it issues loads (the CU's
-  // vector memory path takes 64 bytes per cycle and all eight wavefronts queue up).  K(i+3) and V(i+2) are issued
-  // after Y(i), at the end of the softmax phase, or (d = 64) inside the MFMA phase that follows it; both stages were
-  // last read in tick 2i-1.  Issue order per wavefront: K0 V0 | K1 K2 V1 | K3 V2 | K4 V3 | ...
-  // The odd barriers are left out (not with FULLP): they publish nothing - K(m) and V(m-1) are published by barrier
-  // 2m - and a stage is refilled a whole key block after its last read either way.  Between two barriers wavefronts
-  // 0..3 then run M(i) Y(i) and wavefronts 4..7 run Y(i-1) M(i), still in anti-phase, but without meeting in the
-  // middle.  Where the tile loads are not issued inside the MFMA phase (d = 128), wavefronts 0..3 issue theirs right
-  // after the barrier, in front of their MFMA phase, like wavefronts 4..7 do in front of theirs.
-  // FULLP: wavefronts 4..7 sum the columns of V(i+1) inside M(i), before their GEMM 1 of that block, and the sums are
-  // read in M(i+1) by everyone, behind barrier 2i+4.  V therefore runs one key block further ahead than K needs (the
-  // four V stages hold V(i) .. V(i+3)): barrier 2m publishes K(m) and V(m) instead of K(m) and V(m-1), and the first
-  // barrier V(0).  Issue order per wavefront: K0 V0 | K1 V1 K2 V2 | K3 V3 | K4 V4 | ...
-  // (FMHA_TWO_BARRIERS, a test build: the schedule with a barrier between the phases as well, in which barrier 2m+1
-  // publishes the column sums and V runs no further ahead than without FULLP.)
+  // ---- the schedule ------------------------------------------------------------------------------------------------
+  // Every key block i is two phases per wavefront: an MFMA phase M(i) = [P packing and GEMM 2 + merge of block i]
+  // [GEMM 1 of block i+1] and a VALU phase Y(i) = softmax of block i.  The two wavefronts of a SIMD run them in
+  // anti-phase, so that the MFMA phase of one overlaps the VALU phase of the other.  They share one issue port: a key
+  // block lasts about as long as the issue time of both phases of both wavefronts together, and the barrier waits for
+  // the wavefront whose own instruction stream - vector, scalar and memory instructions alike - is the longer one.
+  // ONE workgroup barrier per key block (numbered as the even ones of the two-barrier schedule below): between
+  // barriers 2i+2 and 2i+4 wavefronts 0..3 run M(i) Y(i+1) and wavefronts 4..7 run Y(i) M(i).
+  // Tiles: K(j), V(j) live in stage j mod 4; barrier 2m publishes K(m) and V(m-1), the operands of M(m-1) behind it.  K(i+3) and V(i+2) are requested inside M(i), one load behind each output
+  // tile of GEMM 2 (a wavefront that issues loads is held for hundreds of cycles - the CU's vector memory path takes
+  // 64 bytes per cycle and all eight wavefronts queue up - and there the hold falls into the waits of the MFMA chain);
+  // their stages held K(i-1) and V(i-2), last read in M(i-2), which ends before barrier 2i.  Issue order per
+  // wavefront: K0 V0 | K1 K2 V1 | K3 V2 | K4 V3 | ...
+  // FULLP at d = 128: wavefronts 4..7 sum the columns of V(i+1) inside M(i), before their GEMM 1 of that block, and
+  // the sums are read in M(i+1) by everyone, behind barrier 2i+4.  V therefore runs one key block further ahead than K
+  // needs (the four V stages hold V(i) .. V(i+3)): barrier 2m publishes K(m) and V(m) instead of K(m) and V(m-1), and
+  // the first barrier V(0).  Issue order per wavefront: K0 V0 | K1 V1 K2 V2 | K3 V3 | K4 V4 | ...
+  // TWO barriers per key block (FULLP at d = 64, and the test build FMHA_TWO_BARRIERS): a tick is the interval between
+  // two barriers; wavefronts 0..3 run M in even ticks and Y in odd ones, wavefronts 4..7 one tick behind.  The odd
+  // barriers publish no tile; with FULLP barrier 2m+1 publishes the column sums of V(m), taken in tick 2m+1, and V runs
+  // no further ahead than without FULLP.  Where the tile loads are not issued inside the MFMA phase (the staged test
+  // build), wavefronts 0..3 issue theirs right after the barrier, in front of their MFMA phase, like wavefronts 4..7.
   auto barrier_odd = [&]() { if (!kOneBarrier) barrier(); };
   const int n = kb_end;
   auto cls_of = [&](int kb) { return __builtin_amdgcn_readfirstlane((int)lds_class[kb]); };
