@@ -90,6 +90,8 @@ __device__ __forceinline__ constexpr bool fmha_in_bounds(bool) { return true; }
 //   FMHA_KO_SOFTMAX      the block softmax is not computed (P, block maximum and row sum are left undefined)
 //   FMHA_KO_MFMA         GEMM 2 + merge and GEMM 1 + row maximum are not computed (with FMHA_KO_SOFTMAX: the key loop
 //                        is tile loads, waits and barriers only)
+//   FMHA_KO_SCALE_RUN, FMHA_KO_EXP_RUN, FMHA_KO_SUM_RUN   one of the three dense runs of the steady-state softmax is
+//                        left out: the 64 scale fmas (and conversions), the 64 exponentials, the 64 + 4 row-sum adds
 //   FMHA_KO_LDS_READS    the MFMA operands are undefined registers instead of LDS reads
 //   FMHA_KO_TILE_LOADS   no K/V tile is fetched after the prologue
 //   FMHA_NO_SWIZZLE      K and V tiles lie in LDS as plain [key][d] rows (results unchanged, bank conflicts are not)
@@ -614,23 +616,33 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #pragma unroll
         for (int qd = 0; qd < kQuads; ++qd)
 #pragma unroll
+#ifdef FMHA_KO_SCALE_RUN
+          for (int j = 0; j < 4; ++j) xs[qd][j] = __int_as_float(acc[qd / 4][4 * (qd % 4) + j]);
+#else
           for (int j = 0; j < 4; ++j) xs[qd][j] = __builtin_fmaf(sf(qd / 4, 4 * (qd % 4) + j), c2, -offq);
+#endif
 #pragma unroll
         for (int qd = 0; qd < kQuads; ++qd) asm volatile("" : "+v"(xs[qd][0]), "+v"(xs[qd][1]), "+v"(xs[qd][2]), "+v"(xs[qd][3]));
         __builtin_amdgcn_sched_barrier(0);
+#ifndef FMHA_KO_EXP_RUN
 #pragma unroll
         for (int qd = 0; qd < kQuads; ++qd)
 #pragma unroll
           for (int j = 0; j < 4; ++j) xs[qd][j] = __builtin_amdgcn_exp2f(xs[qd][j]);
+#endif
 #pragma unroll
         for (int qd = 0; qd < kQuads; ++qd) asm volatile("" : "+v"(xs[qd][0]), "+v"(xs[qd][1]), "+v"(xs[qd][2]), "+v"(xs[qd][3]));
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int qd = 0; qd < kQuads; ++qd) {
+#ifdef FMHA_KO_SUM_RUN
+          if (qd == 0) l_blk += xs[0][0];
+#else
           float s01 = xs[qd][0] + xs[qd][1];
           const float s23 = xs[qd][2] + xs[qd][3];
           s01 += s23;
           l_blk += s01;
+#endif
 #pragma unroll
           for (int j = 0; j < 4; ++j) acc[qd / 4][4 * (qd % 4) + j] = __float_as_int(xs[qd][j]);
         }
