@@ -40,12 +40,13 @@
 #define OP_PERM(r) "v_perm_b32 v" S_(r) ", v" S_(r) ", v101, v102\n\t"
 #define OP_CVT(r) "v_cvt_f32_i32_e32 v" S_(r) ", v" S_(r) "\n\t"
 #define OP_EXP(r) "v_exp_f32_e32 v" S_(r) ", v" S_(r) "\n\t"
+#define OP_EXPH(r) "v_exp_f16_e32 v" S_(r) ", v" S_(r) "\n\t"
 // 32 MFMAs per 192 slots (two alternating accumulator tiles): the matrix pipe is then busy all the time
 #define MF_(a) "v_mfma_i32_32x32x32_i8 v[" S_(a) ":" S_(a) "+15], v[104:107], v[108:111], v[" S_(a) ":" S_(a) "+15]\n\t"
 #define MF4 MF_(0) MF_(16) MF_(0) MF_(16)
 #define MF32 MF4 MF4 MF4 MF4 MF4 MF4 MF4 MF4
 
-enum Op { kNone, kAdd, kAddS, kMul, kFma, kFmaS, kFmac, kMov, kMax3, kMaxF, kPknorm, kPerm, kCvt, kExp, kMfma, kFmaMis, kPknormMis, kAddMis, kMfmaMis };
+enum Op { kNone, kAdd, kAddS, kMul, kFma, kFmaS, kFmac, kMov, kMax3, kMaxF, kPknorm, kPerm, kCvt, kExp, kExpH, kMfma, kFmaMis, kPknormMis, kAddMis, kMfmaMis };
 #define CLOBBER "memory", "s20", "s21", "v0", "v1", "v2", "v3", "v4", "v5", "v6", "v7", "v8", "v9", "v10", "v11", "v12", "v13", \
     "v14", "v15", "v16", "v17", "v18", "v19", "v20", "v21", "v22", "v23", "v24", "v25", "v26", "v27", "v28", "v29", "v30",     \
     "v31", "v64", "v65", "v66", "v67", "v68", "v69", "v70", "v71", "v100", "v101", "v102", "v104", "v105", "v106", "v107",   \
@@ -74,6 +75,7 @@ __device__ __forceinline__ void stream() {
   if (OP == kPerm) asm volatile(AL R192(OP_PERM) ::: CLOBBER);
   if (OP == kCvt) asm volatile(AL R192(OP_CVT) ::: CLOBBER);
   if (OP == kExp) asm volatile(AL R192(OP_EXP) ::: CLOBBER);
+  if (OP == kExpH) asm volatile(AL R192(OP_EXPH) ::: CLOBBER);
   if (OP == kMfma) asm volatile(AL MF32 ::: CLOBBER);
 }
 
@@ -126,6 +128,7 @@ int main(int argc, char** argv) {
   ROW(kFma, kNone, kNone, "v_fma_f32 alone");
   ROW(kMax3, kNone, kNone, "v_max3_i32 alone");
   ROW(kExp, kNone, kNone, "v_exp_f32 alone");
+  ROW(kExpH, kNone, kNone, "v_exp_f16 alone");
   printf("# -- the same from an address that is 4 mod 8: a 64-bit encoding then straddles two aligned dword pairs\n");
   ROW(kAddMis, kNone, kNone, "v_add_f32 (32-bit encoding) alone, at 4 mod 8");
   ROW(kFmaMis, kNone, kNone, "v_fma_f32 (64-bit encoding) alone, at 4 mod 8");
