@@ -15,8 +15,6 @@
 //                          many MiB of fp32 input, checked bit for bit against the CPU checker and timed against HBM
 //   --calibrate-copy MiB   also run one device-to-device copy of that size, so that a counter run (FETCH_SIZE /
 //                          WRITE_SIZE) sees a plain copy kernel of known traffic to scale the attention kernel's by
-//   --lds-patterns         run the LDS operand-read microbenchmark that sits beside this binary (tests/lds_patterns.hip:
-//                          the K and V read patterns with and without the swizzle) as a child process and exit with its code
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
@@ -27,8 +25,6 @@
 #include <string>
 #include <vector>
 
-#include <spawn.h>
-#include <sys/wait.h>
 #include <unistd.h>
 
 #include "fmha_i8.h"
@@ -438,24 +434,6 @@ int main(int argc, char** argv) {
     else if (a == "--json") opt.json = val();
     else if (a == "--calibrate-copy") calib_mib = atol(val());
     else if (a == "--quant") quant_mib = atol(val());
-    else if (a == "--lds-patterns") {
-      // a child process (never an exec from a process that may already hold the GPU), before any HIP call of ours
-      std::string self(4096, '\0');
-      const ssize_t len = readlink("/proc/self/exe", &self[0], self.size() - 1);
-      if (len <= 0) return 2;
-      self.resize(len);
-      const std::string tool = self.substr(0, self.rfind('/') + 1) + "lds_patterns";
-      char* child_argv[] = {const_cast<char*>(tool.c_str()), nullptr};
-      pid_t pid;
-      extern char** environ;
-      if (posix_spawn(&pid, tool.c_str(), nullptr, nullptr, child_argv, environ) != 0) {
-        fprintf(stderr, "cannot start %s (make -C tests all builds it)\n", tool.c_str());
-        return 2;
-      }
-      int status = 0;
-      waitpid(pid, &status, 0);
-      return WIFEXITED(status) ? WEXITSTATUS(status) : 1;
-    }
     else {
       fprintf(stderr, "unknown argument %s\n", a.c_str());
       return 2;
