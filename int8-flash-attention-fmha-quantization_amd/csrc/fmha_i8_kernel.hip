@@ -199,6 +199,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   __shared__ unsigned char lds_class[kMaxKeyBlocks];  // per key block: bit0 = some key masked, bit1 = all keys masked
   __shared__ unsigned lds_mask[kMaxKeyBlocks * kBlockKSmall / 32];  // bit j%32 of word j/32: key j of this batch entry is masked
   __shared__ __attribute__((aligned(16))) int lds_colsum[FULLP ? 2 * D : 4];  // FULLP: [key block & 1][output column]
+  __shared__ __attribute__((aligned(16))) int lds_scan[8];  // per classifying wavefront: last block with an unmasked key, first block with a masked one
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -271,13 +272,14 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // LDS-DMA builtin as a store that may alias every later LDS read and would wait for tiles that are still in flight
   // before the first operand read of the current one.  Completion is tracked by hand with s_waitcnt vmcnt(n) in front
   // of the barrier that publishes a tile.  M0 carries the LDS destination of lane 0; lane l lands 16*l bytes further.
+  // (M0 cannot be named as a clobber: the compiler reserves it and rejects it on a clobber list.  Every statement here
+  // that needs M0 sets it itself, in the same statement, so none depends on what another one left there.)
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) int8_t*)&lds[0][0][0];
   // Tile 0 of a sequence shorter than one block - the only tile there is, fetched in the prologue and again at every
   // later issue point: rows past the last key fetch the last key instead (same chunk: the swizzle belongs to the LDS
   // row); what lands there is never attended to, those keys are masked.  Fetching the whole tile would read up to
   // BK - S rows past the end of K and V.
-  auto issue_short_region = [&](const int8_t* gbase, int which, int goff, int it) {
-    const int region = (it * kWaves + wave) % kRegions;
+  auto issue_short_region = [&](const int8_t* gbase, int which, int goff, int region) {
     const unsigned dst = lds_base + (unsigned)(which * kTileBytes + region * 1024);
     const int row = region * kRowsPerRegion + ld_row_in;
     int src = goff + region * 1024 - (row >= S ? (row - (S - 1)) * D : 0);
@@ -290,13 +292,13 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #ifdef FMHA_KO_TILE_LOADS
     if (prologue_done) return;
 #endif
+    const int region = (it * kWaves + wave) % kRegions;
     if (RAGGED && short_seq) {
-      issue_short_region(gbase, which, goff, it);
+      issue_short_region(gbase, which, goff, region);
       return;
     }
     const int8_t* gp = gbase + (long)kb * kTileBytes;  // wave-uniform base (SGPR pair)
     if (RAGGED && kb == tail_kb) gp = gbase + (long)(S - BK) * D;
-    const int region = (it * kWaves + wave) % kRegions;
     const unsigned dst = lds_base + (unsigned)(((kb & (kStages - 1)) * 2 + which) * kTileBytes + region * 1024);
     int src = goff + region * 1024;
     {
@@ -305,6 +307,31 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     }
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(dst), "v"(src), "s"(gp) : "memory");
+  };
+  // Region `region` of tile 0 (the prologue, where the tiles are split between the wavefronts differently)
+  auto issue_region0_at = [&](const int8_t* gbase, int which, int goff, int region) {
+    if (RAGGED && short_seq) {
+      issue_short_region(gbase, which, goff, region);
+      return;
+    }
+    const int8_t* gp = gbase;
+    if (RAGGED && tail_kb == 0) gp = gbase + (long)(S - BK) * D;
+    const unsigned dst = lds_base + (unsigned)(which * kTileBytes + region * 1024);
+    int src = goff + region * 1024;
+    {
+      const long rel = (long)(gp - gbase) + src;  // offset inside the head
+      if (!fmha_in_bounds(rel >= 0 && rel + 16 <= (long)S * D)) src = (int)(gbase - gp);
+    }
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(dst), "v"(src), "s"(gp) : "memory");
+  };
+  // Tile 0 in the prologue: K0 is fetched by wavefronts 0..3 alone and V0 by wavefronts 4..7 alone (regions
+  // (wave & 3) + 4 it: the same parity as the wavefront's regions in the key loop, which the swizzled offsets assume),
+  // so that the first barrier, which publishes K0, does not wait for the wavefronts that start last.
+  constexpr int kPrologueRegions = (kRegions + 3) / 4;
+  auto issue_tile0_by_half = [&](const int8_t* gbase, int which, int goff) {
+#pragma unroll
+    for (int it = 0; it < kPrologueRegions; ++it) issue_region0_at(gbase, which, goff, (4 * it + (wave & 3)) % kRegions);
   };
   auto issue_tile = [&](const int8_t* gbase, int kb, int which, int goff) {
 #pragma unroll
@@ -328,6 +355,19 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // behind them fall (+12 % when they straddle), so it pins those, the scale fmas and the P packing to aligned
   // addresses; the d = 128 kernel measures the same either way (+-0.3 %) and is left alone.
   auto align8 = [&]() { if (D == 64) asm volatile(".p2align 3" ::: "memory"); };
+  // The steady-state loops start at a fixed distance from a 64-byte boundary, so that what is measured for them does
+  // not change with the code in front of them: at d = 64 the loop of wavefronts 0..3 runs 12 % slower when it starts
+  // 4 bytes further on or back (B16 H16 S2048: 226 against 254 us; every even distance measures the same, every odd
+  // one too; the loop of wavefronts 4..7 measures the same either way, and so do both loops at d = 128).  What flips
+  // with those 4 bytes is whether the eight v_max3_i32 at the top of the loop - the first readers of the last MFMA of
+  // GEMM 1 - start at 8-byte-aligned addresses (fast) or straddle two (slow).  The right distance is found by timing
+  // (tests/variant_timing.py, -DFMHA_LOOP_PAD_A=0 against 1) whenever the code between the boundary and the loop changes.
+  auto align_loop = [&]() { asm volatile(".p2align 6" ::: "memory"); };
+#ifdef FMHA_LOOP_PAD_A
+  constexpr int kLoopPadA = FMHA_LOOP_PAD_A;
+#else
+  constexpr int kLoopPadA = D == 64 ? 1 : 0;  // s_nops between the boundary and the loop of wavefronts 0..3 (see above)
+#endif
 #ifdef FMHA_TRACE_TICKS
   unsigned trace_reg = 0;
   int trace_n = 0;
@@ -361,22 +401,54 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #endif
   constexpr int kVAhead = (FULLP && kOneBarrier) ? 3 : 2;
 
-  // Loads of the prologue, all issued before any is waited for and all by inline assembly, so that every wait is an
-  // explicit s_waitcnt vmcnt(n) that counts the loads still allowed in flight (memory reads return in issue order):
-  //   mask bytes of the first 2048 keys (1 load) | K0 | Q (kDSteps loads) | V0
-  // (the next tiles follow right after the first barrier: the CU's vector memory path moves 64 bytes per cycle, and
-  // everything queued here delays the first GEMM.)
   const int row0 = qb * kBlockQ + wave * 32;  // first query row of this wavefront
   const bool active = row0 < Sq;              // the last workgroup of a head may be partly empty
-  int mask_word = 0;
-  if (!RAGGED || S >= 4) {  // (a shorter mask row has no dword that lies inside it)
-    int j = 4 * tid + 4 <= S ? 4 * tid : S - 4;
-    if (!fmha_in_bounds(j >= 0 && j + 4 <= S)) j = 0;
-    asm volatile("global_load_dword %0, %1, %2" : "=v"(mask_word) : "v"(j), "s"(mg) : "memory");
-  }
-  issue_k(0);
-  v4i qreg[kDSteps];  // Q: B operand of GEMM 1, loaded once
-  {
+
+  // ---- state of a wavefront ----------------------------------------------------------------------------------------
+  // (declared here, ahead of the code that uses it; given its start values by init_state(), which each half of the
+  // workgroup calls once its first loads are on their way)
+  float o_f[kDSteps][16];  // running O, not normalised
+  float m_ref;             // reference exponent of the running O and l (base-2 units)
+  float t_run;             // FASTACC: sum of the merge weights, i.e. how much of kBase the running O carries
+  float l_run;             // running row sum, in units of 1/128 (it sums 128*p)
+  const float c2 = BIAS ? args.c2 * kBaseScale : args.c2;  // exponent per unit of sf() below
+  const float bias_c2 = BIAS ? kBase * c2 : 0.f;
+  float magic;
+  int flip_top;
+  v16i base_c;
+  v4i qreg[kDSteps];       // Q: B operand of GEMM 1, loaded once
+  int kb_end = 0;          // one past the last key block that holds any unmasked key (trailing padding is never computed on)
+  int kb_plain = 0;        // the first block with any masked key: blocks [0, kb_plain) have none
+  int n = 0, last = -1;    // kb_end and kb_end - 1 under the names the schedule uses
+  unsigned tail_word[kKeyTiles];  // RAGGED: mask bits of the shifted last block
+  auto init_state = [&]() {
+#pragma unroll
+    for (int u = 0; u < kDSteps; ++u)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o_f[u][r] = 0.f;
+    m_ref = args.floor2 - 2.f * kLazyLog2;
+    t_run = 0.f;
+    l_run = 0.f;
+    magic = kMagic;
+    asm volatile("" : "+v"(magic));  // a register operand: as a literal it would double the size of every instruction using it
+    flip_top = (int)0x80808080;
+    if (FULLP) asm volatile("" : "+s"(flip_top));  // a register operand, for the same reason
+    base_c = v16i{kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits,
+                  kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits};
+    asm volatile("" : "+v"(base_c));  // held in registers: as a known constant it is rebuilt by eight moves per key block
+  };
+
+  // ---- the prologue ------------------------------------------------------------------------------------------------
+  // Its loads are all issued before any is waited for and all by inline assembly, so that every wait is an explicit
+  // s_waitcnt vmcnt(n) that counts the loads still allowed in flight (memory reads return in issue order):
+  //   wavefronts 0..3:  K0 (all of it) | mask bytes of the first 4096 keys (1 load) | Q (kDSteps loads)
+  //   wavefronts 4..7:  Q (kDSteps loads) | behind the first barrier: V0 (all of it)
+  // (the next tiles follow right after the first barrier: the CU's vector memory path moves 64 bytes per cycle, and
+  // everything queued here delays the first GEMM.)  The first barrier publishes K0, which wavefronts 0..3 fetch alone:
+  // it waits for nothing that wavefronts 4..7, which start several hundred cycles later, have asked for.  Each half of
+  // the workgroup runs its own prologue and its own schedule behind ONE branch on the wavefront index, so that a load
+  // and the wait that retires it always lie on the same path.
+  auto load_q_rows = [&]() {
     // rows past the end of the sequence load the last row (unused) so that every wavefront has the same loads in flight
     const int8_t* qp = args.q + q_head_off;
     int qrow = row0 + i32 < Sq ? row0 + i32 : Sq - 1;
@@ -385,95 +457,138 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #pragma unroll
     for (int kk = 0; kk < kDSteps; ++kk)
       asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(qreg[kk]) : "v"(qoff + 32 * kk), "s"(qp) : "memory");
-  }
-  issue_v(0);
-
-  // ---- classify the key blocks of this batch entry: 4 mask bytes per lane, BK/4 lanes per block ---------------------
-  asm volatile("s_waitcnt vmcnt(%1)" : "+v"(mask_word) : "n"(2 * kRegionsPerWave + kDSteps) : "memory");
-  for (int base = 0; base < S_pad; base += 4 * kThreads) {
-    const int j = base + 4 * tid;
-    int nib = 15;  // keys past the end of the sequence count as masked
-    if (RAGGED ? j + 4 <= S : j < S) {
-      if (base == 0) {
-        const unsigned w = (unsigned)mask_word;
-        nib = ((w & 0xffu) ? 1 : 0) | ((w & 0xff00u) ? 2 : 0) | ((w & 0xff0000u) ? 4 : 0) | ((w & 0xff000000u) ? 8 : 0);
-      } else {
-        const int jj = fmha_in_bounds(j >= 0 && j + 4 <= S) ? j : 0;
-        nib = (mg[jj] != 0 ? 1 : 0) | (mg[jj + 1] != 0 ? 2 : 0) | (mg[jj + 2] != 0 ? 4 : 0) | (mg[jj + 3] != 0 ? 8 : 0);
+  };
+  // The Q registers are redefined after the wait that retires their loads, so that no use of them can be scheduled
+  // above it.
+  auto pin_q_rows = [&]() {
+#pragma unroll
+    for (int kk = 0; kk < kDSteps; ++kk) asm volatile("" : "+v"(qreg[kk]));
+  };
+  // Wavefronts 0..3 also classify the key blocks of this batch entry, sixteen mask bytes per lane and BK/16 lanes per
+  // block: their loads are the first to be served.  Per key block: lds_class (bit0 = some key masked, bit1 = all keys
+  // masked) and the mask bits themselves (lds_mask); per classifying wavefront: the last block it saw with an unmasked
+  // key and the first with a masked one (lds_scan).  All of it is published by the first barrier, together with K0.
+  constexpr int kClassWaves = 4;
+  constexpr int kKeysPerLane = 16;
+  constexpr int kKeysPerPass = kKeysPerLane * 64 * kClassWaves;
+  auto prologue_waves_0_to_3 = [&]() {
+    issue_tile0_by_half(kg, 0, ld_goff_k);
+    v4i mask_bytes = {0, 0, 0, 0};
+    {
+      const bool inside = kKeysPerLane * tid + kKeysPerLane <= S;
+      int j = inside ? kKeysPerLane * tid : 0;
+      if (!fmha_in_bounds(!inside || (j >= 0 && j + kKeysPerLane <= S))) j = 0;
+      if (!RAGGED || S >= kKeysPerLane)  // (a shorter mask row has no 16 bytes that lie inside it)
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(mask_bytes) : "v"(j), "s"(mg) : "memory");
+    }
+    load_q_rows();
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(mask_bytes) : "n"(kDSteps) : "memory");
+    constexpr int kLanesPerBlock = BK / kKeysPerLane;
+    constexpr int kBlocksPerWave = 64 / kLanesPerBlock;
+    constexpr unsigned long long kGroupBits = kLanesPerBlock == 8 ? 0x0101010101010101ull : 0x1111111111111111ull;
+    int live_hi = -1, pad_lo = 0x7fffffff;
+    // one bit per byte of a dword: set where the byte is not zero
+    auto nonzero_bytes = [](unsigned w) -> unsigned {
+      const unsigned t = (((w & 0x7f7f7f7fu) + 0x7f7f7f7fu) | w) & 0x80808080u;  // bit 7 of every nonzero byte
+      return (((t >> 7) * 0x00204081u) >> 21) & 15u;                           // ... gathered into bits 0..3
+    };
+    for (int base = 0; base < S_pad; base += kKeysPerPass) {
+      const int j = base + kKeysPerLane * tid;
+      unsigned bits = 0xffffu;  // keys past the end of the sequence count as masked
+      if (j + kKeysPerLane <= S) {
+        v4i w = mask_bytes;
+        if (base != 0) {
+          const int jj = fmha_in_bounds(j >= 0 && j + kKeysPerLane <= S) ? j : 0;
+          asm volatile("global_load_dwordx4 %0, %1, %2\n\ts_waitcnt vmcnt(0)" : "=v"(w) : "v"(jj), "s"(mg) : "memory");
+        }
+        bits = nonzero_bytes((unsigned)w[0]) | (nonzero_bytes((unsigned)w[1]) << 4) | (nonzero_bytes((unsigned)w[2]) << 8) |
+               (nonzero_bytes((unsigned)w[3]) << 12);
+      } else if (RAGGED && j < S) {  // the one lane that straddles the end
+        for (int b = 0; b < S - j; ++b) bits = (mg[fmha_in_bounds(j + b < S) ? j + b : 0] != 0) ? bits : (bits & ~(1u << b));
       }
-    } else if (RAGGED && j < S) {  // the one lane that straddles the end
-      for (int b = 0; b < S - j; ++b) nib = (mg[fmha_in_bounds(j + b < S) ? j + b : 0] != 0) ? nib : (nib & ~(1 << b));
+      // two lanes hold the 32 mask bits of one word
+      const unsigned word = bits | ((unsigned)__shfl_xor((int)bits, 1) << 16);
+      if ((lane & 1) == 0 && j < S_pad) lds_mask[j >> 5] = word;
+      const unsigned long long some = __ballot(bits != 0), all = __ballot(bits == 0xffffu);
+      if (lane % kLanesPerBlock == 0 && j < S_pad) {
+        constexpr unsigned long long kBlockBits = (1ull << kLanesPerBlock) - 1;
+        const unsigned long long blk_some = (some >> lane) & kBlockBits, blk_all = (all >> lane) & kBlockBits;
+        lds_class[j / BK] = (unsigned char)((blk_some != 0 ? 1 : 0) | (blk_all == kBlockBits ? 2 : 0));
+      }
+      // the same two facts per block of this wavefront, folded onto the lowest lane of each block (wave-uniform)
+      unsigned long long any = some, every = all;
+#pragma unroll
+      for (int sh = 1; sh < kLanesPerBlock; sh *= 2) {
+        any |= any >> sh;
+        every &= every >> sh;
+      }
+      const int blk0 = (base + kKeysPerLane * 64 * wave) / BK;  // first block of this wavefront in this pass
+      const int n_here = min(max(n_blocks - blk0, 0), kBlocksPerWave);
+      const unsigned long long valid = (n_here == kBlocksPerWave ? ~0ull : ((1ull << (n_here * kLanesPerBlock)) - 1ull)) & kGroupBits;
+      const unsigned long long live = ~every & valid, padded = any & valid;
+      if (live != 0) live_hi = blk0 + (63 - __builtin_clzll(live)) / kLanesPerBlock;
+      if (padded != 0) pad_lo = min(pad_lo, blk0 + __builtin_ctzll(padded) / kLanesPerBlock);
     }
-    // eight lanes hold the 32 mask bits of one word
-    unsigned word = (unsigned)nib << (4 * (lane & 7));
-    word |= __shfl_xor(word, 1);
-    word |= __shfl_xor(word, 2);
-    word |= __shfl_xor(word, 4);
-    if ((lane & 7) == 0 && j < S_pad) lds_mask[j >> 5] = word;
-    const unsigned long long some = __ballot(nib != 0), all = __ballot(nib == 15);
-    constexpr int kLanesPerBlock = BK / 4;
-    constexpr unsigned long long kBlockBits = (1ull << kLanesPerBlock) - 1;
-    if (lane % kLanesPerBlock == 0 && j < S_pad) {
-      const unsigned long long blk_some = (some >> lane) & kBlockBits, blk_all = (all >> lane) & kBlockBits;
-      lds_class[j / BK] = (unsigned char)((blk_some != 0 ? 1 : 0) | (blk_all == kBlockBits ? 2 : 0));
+    if (lane == 0) {
+      lds_scan[2 * wave] = live_hi;
+      lds_scan[2 * wave + 1] = pad_lo;
     }
-  }
-  __syncthreads();
-  // mask bits of the shifted last block: bit r of word t <-> key S - BK + 32 t + r; the repeated keys count as masked
-  unsigned tail_word[kKeyTiles];
-#pragma unroll
-  for (int t = 0; t < kKeyTiles; ++t) tail_word[t] = 0;
-  if (RAGGED && tail_kb >= 0) {
-    const int repeated = BK - tail_rows;
-#pragma unroll
-    for (int t = 0; t < kKeyTiles; ++t) {
-      const int start = S - BK + 32 * t, w = start >> 5, sh = start & 31;
-      const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_mask[w]);
-      const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_mask[w + (sh ? 1 : 0)]);
-      unsigned word = sh ? (lo >> sh) | (hi << (32 - sh)) : lo;
-      const int forced = repeated - 32 * t;  // leading bits of this word that belong to repeated keys
-      if (forced >= 32) word = 0xffffffffu;
-      else if (forced > 0) word |= (1u << forced) - 1u;
-      tail_word[t] = word;
+    init_state();
+    // K0 and the Q rows have landed; the LDS writes above are not waited for by the hand-written barrier
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    pin_q_rows();
+  };
+  // Wavefronts 4..7 ask for their Q rows only and wait for nothing in front of the first barrier; right behind it they
+  // wait for the Q rows (their first GEMM 1 comes one phase later anyway) and then ask for V0, which is first needed
+  // behind the second barrier.  Every wait of the prologue is a vmcnt(0): it holds on whatever path leads to it.
+  // (FULLP with one barrier per key block: V0 in front of the first barrier - they sum its columns right behind it.)
+  constexpr bool kV0BeforeFirstBarrier = FULLP && kOneBarrier;
+  auto prologue_waves_4_to_7 = [&]() {
+    load_q_rows();
+    if (kV0BeforeFirstBarrier) issue_tile0_by_half(vg, 1, ld_goff_v);
+    init_state();
+    if (kV0BeforeFirstBarrier) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      pin_q_rows();
     }
-  }
-  // last key block that holds any unmasked key (trailing padding is never computed on)
-  int last_block = -1, first_padded = n_blocks;  // (and the first block with any masked key)
-  for (int base = 0; base < n_blocks; base += 64) {
-    const int blk = base + lane;
-    const int c = lds_class[blk < n_blocks ? blk : 0];
-    const unsigned long long live = __ballot(blk < n_blocks && !(c & 2));
-    const unsigned long long padded = __ballot(blk < n_blocks && c != 0);
-    if (live != 0) last_block = base + 63 - __builtin_clzll(live);
-    if (padded != 0 && first_padded == n_blocks) first_padded = base + __builtin_ctzll(padded);
-  }
-  const int kb_end = __builtin_amdgcn_readfirstlane(last_block) + 1;
-  const int kb_plain = __builtin_amdgcn_readfirstlane(first_padded);  // blocks [0, kb_plain) have no masked key
-
-  float o_f[kDSteps][16];
+  };
+  auto q_rows_landed_then_v0 = [&]() {  // wavefronts 4..7, behind the first barrier
+    if (!kV0BeforeFirstBarrier) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      pin_q_rows();
+      issue_tile0_by_half(vg, 1, ld_goff_v);
+    }
+  };
+  // Barrier 0 publishes K0, the block classes, the mask bits and the scan records; every wavefront then reads what the
+  // classification found.
+  auto first_barrier = [&]() {
+    prologue_done = true;
+    barrier();
+    {
+      const v4i s0 = *reinterpret_cast<const v4i*>(&lds_scan[0]), s1 = *reinterpret_cast<const v4i*>(&lds_scan[4]);
+      kb_end = __builtin_amdgcn_readfirstlane(max(max(s0[0], s0[2]), max(s1[0], s1[2]))) + 1;
+      kb_plain = __builtin_amdgcn_readfirstlane(min(min(min(s0[1], s0[3]), min(s1[1], s1[3])), n_blocks));
+    }
+    n = kb_end;
+    last = n - 1;
+    // mask bits of the shifted last block: bit r of word t <-> key S - BK + 32 t + r; the repeated keys count as masked
 #pragma unroll
-  for (int u = 0; u < kDSteps; ++u)
+    for (int t = 0; t < kKeyTiles; ++t) tail_word[t] = 0;
+    if (RAGGED && tail_kb >= 0) {
+      const int repeated = BK - tail_rows;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) o_f[u][r] = 0.f;
-  float m_ref = args.floor2 - 2.f * kLazyLog2;  // reference exponent of the running O and l (base-2 units)
-  float t_run = 0.f;  // FASTACC: sum of the merge weights, i.e. how much of kBase the running O carries
-  float l_run = 0.f;                            // running row sum, in units of 1/128 (it sums 128*p)
-  const float c2 = BIAS ? args.c2 * kBaseScale : args.c2;  // exponent per unit of sf() below
-  const float bias_c2 = BIAS ? kBase * c2 : 0.f;
-  float magic = kMagic;
-  asm volatile("" : "+v"(magic));  // a register operand: as a literal it would double the size of every instruction using it
-  int flip_top = (int)0x80808080;
-  if (FULLP) asm volatile("" : "+s"(flip_top));  // a register operand, for the same reason
-  v16i base_c = {kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits,
-                 kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits};
-  asm volatile("" : "+v"(base_c));  // held in registers: as a known constant it is rebuilt by eight moves per key block
-
-  // K0 and Q have landed once at most V0 is still in flight.  The registers are redefined after the wait so that no
-  // use of them can be scheduled above it.
-  // (FULLP: V0 as well - wavefronts 4..7 sum its columns right after the first barrier.)
-  asm volatile("s_waitcnt vmcnt(%0)" :: "n"(FULLP && kOneBarrier ? 0 : kRegionsPerWave) : "memory");
-#pragma unroll
-  for (int kk = 0; kk < kDSteps; ++kk) asm volatile("" : "+v"(qreg[kk]));
+      for (int t = 0; t < kKeyTiles; ++t) {
+        const int start = S - BK + 32 * t, w = start >> 5, sh = start & 31;
+        const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_mask[w]);
+        const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_mask[w + (sh ? 1 : 0)]);
+        unsigned word = sh ? (lo >> sh) | (hi << (32 - sh)) : lo;
+        const int forced = repeated - 32 * t;  // leading bits of this word that belong to repeated keys
+        if (forced >= 32) word = 0xffffffffu;
+        else if (forced > 0) word |= (1u << forced) - 1u;
+        tail_word[t] = word;
+      }
+    }
+  };
 
   // ---- the four phases of one key block ----------------------------------------------------------------------------
   // acc:  S^T, for query column i32 keys 32t + 8a + 4g + bb at acc[t][4a+bb]        (GEMM 1 -> softmax)
@@ -886,14 +1001,12 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // no further ahead than without FULLP.  Where the tile loads are not issued inside the MFMA phase (the staged test
   // build), wavefronts 0..3 issue theirs right after the barrier, in front of their MFMA phase, like wavefronts 4..7.
   auto barrier_odd = [&]() { if (!kOneBarrier) barrier(); };
-  const int n = kb_end;
   auto cls_of = [&](int kb) { return __builtin_amdgcn_readfirstlane((int)lds_class[kb]); };
   auto works = [&](int kb) { return active && !(cls_of(kb) & 2); };  // nothing in a fully masked block is attended to
   // Every issue point issues the same number of tiles whatever the position in the sequence: a tile index past the
   // last block is replaced by the last block, which is then fetched again into the stage it already occupies (the
   // same bytes: harmless for the wavefronts reading it).  That keeps the wait counts below compile-time constants and
   // the key loop free of the compares and branches that a count depending on the position would need.
-  const int last = n - 1;
   auto issue_first = [&]() {          // after barrier 0
     if (n > 0) {
       if (FULLP && kOneBarrier) {  // in pairs, so that "all but the newest two tiles" means the same at every barrier
@@ -986,9 +1099,9 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // that waits behind the other wavefront's softmax stream leaves the MFMA pipe idle, the reverse costs nothing.
   auto raise_priority = [&]() { asm volatile("s_setprio 3" ::: "memory"); };
   auto drop_priority = [&]() { asm volatile("s_setprio 0" ::: "memory"); };
-  prologue_done = true;
-  barrier();                                   // barrier 0 (K(0) landed: prologue)
-  if (wave < 4) {
+  if (wave < kClassWaves) {
+    prologue_waves_0_to_3();
+    first_barrier();
     if (n > 0 && works(0)) phase_gemm1(0, acc, mx);
     else forget_scores();
     issue_first();
@@ -997,6 +1110,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     // below with every decision taken (scalar compares and branches are not free: they stand in the issue stream of
     // the wavefront that the barrier is waiting for).
     if (active) {
+      align_loop();
+      asm volatile(".rept %0\n\ts_nop 0\n\t.endr" :: "n"(kLoopPadA) : "memory");
       for (; i + 1 < n && i + 1 < kb_plain; ++i) {
         v4i pk[kKeyTiles];
         wait_v_for_colsum_a();
@@ -1043,6 +1158,9 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     }
     barrier_odd();                             // barrier 2n+1: wavefronts 4..7 run their last MFMA phase after it
   } else {
+    prologue_waves_4_to_7();
+    first_barrier();
+    q_rows_landed_then_v0();
     issue_first();
     if (FULLP && !kOneBarrier) wait_all_but(3);  // V(0) has landed: K1 K2 V1 may be in flight
     barrier_odd();                             // barrier 1
@@ -1052,6 +1170,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     if (FULLP) colsum_written();
     int i = 0;
     if (active) {  // steady state, see above
+      align_loop();
       for (; i + 1 < n && i + 1 < kb_plain; ++i) {
         v4i pk[kKeyTiles];
         wait_tiles(false);
