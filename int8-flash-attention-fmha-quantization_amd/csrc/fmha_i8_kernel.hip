@@ -237,6 +237,9 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 
   // The prologue puts every cold miss in flight before it waits for any of them: the mask bytes, the first two K/V
   // tiles (tile 1 on speculation: it exists whenever seq_kv >= 256, whether or not its keys are masked) and the Q rows.
+  // (Every lambda of this kernel that touches the register-resident state - accumulators, running O, Q - is marked
+  // always_inline: one that the compiler decided to call instead would force what it captures by reference into
+  // scratch memory.)
   // ---- per-lane addressing -----------------------------------------------------------------------------------------
   // direct-to-LDS loads: lane l of a 1 KiB region lands at byte 16*l of the region, so the lane FETCHES the chunk that
   // the swizzle assigns to that slot.
@@ -279,7 +282,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // later issue point: rows past the last key fetch the last key instead (same chunk: the swizzle belongs to the LDS
   // row); what lands there is never attended to, those keys are masked.  Fetching the whole tile would read up to
   // BK - S rows past the end of K and V.
-  auto issue_short_region = [&](const int8_t* gbase, int which, int goff, int region) {
+  auto issue_short_region = [&](const int8_t* gbase, int which, int goff, int region) __attribute__((always_inline)) {
     const unsigned dst = lds_base + (unsigned)(which * kTileBytes + region * 1024);
     const int row = region * kRowsPerRegion + ld_row_in;
     int src = goff + region * 1024 - (row >= S ? (row - (S - 1)) * D : 0);
@@ -288,7 +291,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
                  :: "s"(dst), "v"(src), "s"(gbase) : "memory");
   };
   bool prologue_done = false;  // (FMHA_KO_TILE_LOADS)
-  auto issue_region = [&](const int8_t* gbase, int kb, int which, int goff, int it) {  // which: 0 = K, 1 = V
+  auto issue_region = [&](const int8_t* gbase, int kb, int which, int goff, int it) __attribute__((always_inline)) {  // which: 0 = K, 1 = V
 #ifdef FMHA_KO_TILE_LOADS
     if (prologue_done) return;
 #endif
@@ -309,7 +312,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
                  :: "s"(dst), "v"(src), "s"(gp) : "memory");
   };
   // Region `region` of tile 0 (the prologue, where the tiles are split between the wavefronts differently)
-  auto issue_region0_at = [&](const int8_t* gbase, int which, int goff, int region) {
+  auto issue_region0_at = [&](const int8_t* gbase, int which, int goff, int region) __attribute__((always_inline)) {
     if (RAGGED && short_seq) {
       issue_short_region(gbase, which, goff, region);
       return;
@@ -329,16 +332,16 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // (wave & 3) + 4 it: the same parity as the wavefront's regions in the key loop, which the swizzled offsets assume),
   // so that the first barrier, which publishes K0, does not wait for the wavefronts that start last.
   constexpr int kPrologueRegions = (kRegions + 3) / 4;
-  auto issue_tile0_by_half = [&](const int8_t* gbase, int which, int goff) {
+  auto issue_tile0_by_half = [&](const int8_t* gbase, int which, int goff) __attribute__((always_inline)) {
 #pragma unroll
     for (int it = 0; it < kPrologueRegions; ++it) issue_region0_at(gbase, which, goff, (4 * it + (wave & 3)) % kRegions);
   };
-  auto issue_tile = [&](const int8_t* gbase, int kb, int which, int goff) {
+  auto issue_tile = [&](const int8_t* gbase, int kb, int which, int goff) __attribute__((always_inline)) {
 #pragma unroll
     for (int it = 0; it < kRegionsPerWave; ++it) issue_region(gbase, kb, which, goff, it);
   };
-  auto issue_k = [&](int kb) { issue_tile(kg, kb, 0, ld_goff_k); };
-  auto issue_v = [&](int kb) { issue_tile(vg, kb, 1, ld_goff_v); };
+  auto issue_k = [&](int kb) __attribute__((always_inline)) { issue_tile(kg, kb, 0, ld_goff_k); };
+  auto issue_v = [&](int kb) __attribute__((always_inline)) { issue_tile(vg, kb, 1, ld_goff_v); };
   // Memory reads return in issue order: waiting until at most `tiles` tiles of this wavefront's loads are outstanding
   // retires every tile older than the newest `tiles` ones.
   auto wait_all_but = [&](int tiles) {
@@ -421,7 +424,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   int kb_plain = 0;        // the first block with any masked key: blocks [0, kb_plain) have none
   int n = 0, last = -1;    // kb_end and kb_end - 1 under the names the schedule uses
   unsigned tail_word[kKeyTiles];  // RAGGED: mask bits of the shifted last block
-  auto init_state = [&]() {
+  auto init_state = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < kDSteps; ++u)
 #pragma unroll
@@ -448,7 +451,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // it waits for nothing that wavefronts 4..7, which start several hundred cycles later, have asked for.  Each half of
   // the workgroup runs its own prologue and its own schedule behind ONE branch on the wavefront index, so that a load
   // and the wait that retires it always lie on the same path.
-  auto load_q_rows = [&]() {
+  auto load_q_rows = [&]() __attribute__((always_inline)) {
     // rows past the end of the sequence load the last row (unused) so that every wavefront has the same loads in flight
     const int8_t* qp = args.q + q_head_off;
     int qrow = row0 + i32 < Sq ? row0 + i32 : Sq - 1;
@@ -460,7 +463,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   };
   // The Q registers are redefined after the wait that retires their loads, so that no use of them can be scheduled
   // above it.
-  auto pin_q_rows = [&]() {
+  auto pin_q_rows = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int kk = 0; kk < kDSteps; ++kk) asm volatile("" : "+v"(qreg[kk]));
   };
@@ -471,7 +474,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   constexpr int kClassWaves = 4;
   constexpr int kKeysPerLane = 16;
   constexpr int kKeysPerPass = kKeysPerLane * 64 * kClassWaves;
-  auto prologue_waves_0_to_3 = [&]() {
+  auto prologue_waves_0_to_3 = [&]() __attribute__((always_inline)) {
     issue_tile0_by_half(kg, 0, ld_goff_k);
     v4i mask_bytes = {0, 0, 0, 0};
     {
@@ -543,7 +546,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // behind the second barrier.  Every wait of the prologue is a vmcnt(0): it holds on whatever path leads to it.
   // (FULLP with one barrier per key block: V0 in front of the first barrier - they sum its columns right behind it.)
   constexpr bool kV0BeforeFirstBarrier = FULLP && kOneBarrier;
-  auto prologue_waves_4_to_7 = [&]() {
+  auto prologue_waves_4_to_7 = [&]() __attribute__((always_inline)) {
     load_q_rows();
     if (kV0BeforeFirstBarrier) issue_tile0_by_half(vg, 1, ld_goff_v);
     init_state();
@@ -552,7 +555,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       pin_q_rows();
     }
   };
-  auto q_rows_landed_then_v0 = [&]() {  // wavefronts 4..7, behind the first barrier
+  auto q_rows_landed_then_v0 = [&]() __attribute__((always_inline)) {  // wavefronts 4..7, behind the first barrier
     if (!kV0BeforeFirstBarrier) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       pin_q_rows();
@@ -561,7 +564,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   };
   // Barrier 0 publishes K0, the block classes, the mask bits and the scan records; every wavefront then reads what the
   // classification found.
-  auto first_barrier = [&]() {
+  auto first_barrier = [&]() __attribute__((always_inline)) {
     prologue_done = true;
     barrier();
     {
@@ -599,7 +602,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 
   // Row maximum of one finished 32-key tile, folded into two independent chains (integer compare: monotone in the
   // score, also for the biased bit patterns).  Four pieces of two instructions, one behind each MFMA of the next tile.
-  auto tile_max_piece = [&](const v16i& a, int (&mx)[2], bool first, int j) {
+  auto tile_max_piece = [&](const v16i& a, int (&mx)[2], bool first, int j) __attribute__((always_inline)) {
     if (first && j == 0) {
       mx[0] = max(max(a[0], a[1]), a[2]);
       mx[1] = max(max(a[8], a[9]), a[10]);
@@ -614,7 +617,16 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 
   // GEMM 1: S^T[key][query] = K . Q^T, int32 (inc/fmha_i8.cuh:120-172), one 32-key tile after the other; the row
   // maximum of tile t-1 is taken while the MFMAs of tile t run.  mx covers tiles 0 .. kKeyTiles-2 on return.
-  auto phase_gemm1 = [&](int kb, v16i (&acc)[kKeyTiles], int (&mx)[2]) {
+  //
+  // masked = true: some keys of this block are masked out (nonzero mask byte, inc/fmha_i8.cuh:189-192,216-221).  The
+  // ACCUMULATORS of a masked key start at a value that loses every maximum and whose exponential is exactly 0 whatever
+  // the MFMAs add to it - read as a float on the BIAS variant, 0xFF000000 + S is below -2^126 for every |S| < 2^21;
+  // where the scores are converted, -2^30 + S times that variant's c2 >= 2.7e-4 is an exponent below -2.9e5 - so that
+  // the row maximum taken behind the MFMAs and the whole softmax need no further look at the mask.  The start values
+  // are one v_cndmask per score on wave-uniform lane masks - lanes 0..31 hold key 8a+bb of a tile, lanes 32..63 key
+  // 8a+4+bb, so the scalar unit builds them from the block's mask bits - written into the accumulator registers
+  // themselves, tile by tile, in front of the tile's MFMAs.
+  auto phase_gemm1 = [&](int kb, v16i (&acc)[kKeyTiles], int (&mx)[2], bool masked = false) __attribute__((always_inline)) {
 #ifdef FMHA_KO_MFMA
 #pragma unroll
     for (int t = 0; t < kKeyTiles; ++t) asm volatile("" : "=v"(acc[t]));
@@ -629,6 +641,53 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #else
     auto read_k = [&](int off) { return *reinterpret_cast<const v4i*>(lds_k + off); };
 #endif
+    unsigned mw[kKeyTiles];  // masked: the block's mask bits, bit j of word t <-> key 32 t + j of the block
+    int gone = BIAS ? (int)0xFF000000 : -(1 << 30);
+    if (masked) {
+      asm volatile("" : "+v"(gone));  // a register operand
+#pragma unroll
+      for (int t = 0; t < kKeyTiles; ++t)
+        mw[t] = (RAGGED && kb == tail_kb) ? tail_word[t]
+                                          : (unsigned)__builtin_amdgcn_readfirstlane((int)lds_mask[kb * kKeyTiles + t]);
+    }
+    auto start_piece = [&](int t, int first, int count) __attribute__((always_inline)) {  // start values of registers first .. first+count-1 of tile t
+#pragma unroll
+      for (int r = first; r < first + count; ++r) {
+        const int key = 8 * (r / 4) + (r % 4);
+        const unsigned lo = (unsigned)(((int)(mw[t] << (31 - key))) >> 31), hi = (unsigned)(((int)(mw[t] << (27 - key))) >> 31);
+        const unsigned long long lanes = ((unsigned long long)hi << 32) | lo;
+        int e;
+        if (BIAS) asm volatile("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(e) : "v"(base_c[0]), "v"(gone), "s"(lanes));
+        else asm volatile("v_cndmask_b32_e64 %0, 0, %1, %2" : "=v"(e) : "v"(gone), "s"(lanes));
+        acc[t][r] = e;
+      }
+    };
+    if (masked) {
+      // One operand buffer and no read-ahead: the start values of a tile are written while its operand reads are in
+      // flight, and the registers that the read-ahead would take are what the accumulators of the next tile, live one
+      // chain early here, need (with both, the d = 128 kernel spills).
+#pragma unroll
+      for (int t = 0; t < kKeyTiles; ++t) {
+#pragma unroll
+        for (int kk = 0; kk < kDSteps; ++kk) ka[0][kk] = read_k(k_read_off[kk] + 32 * t * D);
+        start_piece(t, 0, 16);
+        asm volatile("s_nop 1" ::: "memory");  // (the compiler does not know that the statements above wrote registers an MFMA reads)
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kk = 0; kk < kDSteps; ++kk) {
+          align8();
+          acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ka[0][kk], qreg[kk], acc[t], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if (t >= 1) {
+#pragma unroll
+            for (int j = kk * 4 / kDSteps; j < (kk + 1) * 4 / kDSteps; ++j) tile_max_piece(acc[t - 1], mx, t == 1, j);
+            asm volatile("" : "+v"(mx[0]), "+v"(mx[1]));
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int kk = 0; kk < kDSteps; ++kk) ka[0][kk] = read_k(k_read_off[kk]);
 #pragma unroll
@@ -659,7 +718,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // split = false: the whole block softmax, P packed, software-pipelined (the general loop).  split = true (the
   // steady-state loop): everything but the P packing, in three dense runs - 64 scale fmas, 64 exponentials, 64 + 4 adds -
   // and the exponentials are left in acc (as float bits) for phase_pack, which runs at the head of the MFMA phase.
-  auto phase_softmax = [&](int kb, int cls, v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles], int (&mx)[2], bool split = false) {
+  auto phase_softmax = [&](int kb, int cls, v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles], int (&mx)[2], bool split = false) __attribute__((always_inline)) {
 #ifdef FMHA_KO_SOFTMAX
     if (!split) {
 #pragma unroll
@@ -670,34 +729,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #endif
     auto sf = [&](int t, int r) -> float { return BIAS ? __int_as_float(acc[t][r]) : (float)acc[t][r]; };
     l_blk = 0.f;
-    if (cls != 0) {
-      // Some keys of this block are masked out (nonzero mask byte, inc/fmha_i8.cuh:189-192,216-221).  Their scores
-      // are replaced by a value that loses every maximum and whose exponential is exactly 0 (-inf read as a float on
-      // the BIAS variant; -2^30 where the scores are converted, which that variant's c2 >= 2.7e-4 turns into an
-      // exponent below -2.9e5), one v_cndmask per score.  The lane masks are wave-uniform - lanes 0..31 hold key
-      // 8a+bb of a tile, lanes 32..63 key 8a+4+bb - so the scalar unit builds them from the block's mask bits.
-      const int gone = BIAS ? (int)0xFF800000 : -(1 << 30);
-#pragma unroll
-      for (int t = 0; t < kKeyTiles; ++t) {
-        const unsigned mw = (RAGGED && kb == tail_kb)
-                                ? tail_word[t]
-                                : (unsigned)__builtin_amdgcn_readfirstlane((int)lds_mask[kb * kKeyTiles + t]);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int key = 8 * (r / 4) + (r % 4);
-          const unsigned lo = (unsigned)(((int)(mw << (31 - key))) >> 31), hi = (unsigned)(((int)(mw << (27 - key))) >> 31);
-          const unsigned long long lanes = ((unsigned long long)hi << 32) | lo;
-          int e = acc[t][r];
-          asm("v_cndmask_b32_e64 %0, %0, %1, %2" : "+v"(e) : "v"(gone), "s"(lanes));
-          acc[t][r] = e;
-        }
-      }
-      // the maximum over the keys that are left (what GEMM 1 collected included the masked ones)
-#pragma unroll
-      for (int t = 0; t + 1 < kKeyTiles; ++t)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) tile_max_piece(acc[t], mx, t == 0, j);
-    }
+    // (cls != 0: some keys of this block are masked out.  GEMM 1 has seen to it that their scores lose every maximum
+    // and that their exponentials are exactly 0; what is left to do here is the reference's sentinel, below.)
     {
 #pragma unroll
       for (int j = 0; j < 4; ++j) tile_max_piece(acc[kKeyTiles - 1], mx, false, j);
@@ -812,7 +845,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     }
   };
   // P packing of the exponentials that phase_softmax(split) left in acc: P^T as the B operand of GEMM 2.
-  auto phase_pack = [&](v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles]) {
+  auto phase_pack = [&](v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles]) __attribute__((always_inline)) {
 #ifdef FMHA_KO_SOFTMAX
 #pragma unroll
     for (int t = 0; t < kKeyTiles; ++t) asm volatile("" : "=v"(pk[t]));
@@ -835,7 +868,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // The steady-state loop uses the split form: -6 % at d = 64 (where it also makes one barrier per key block the faster
   // choice), -2 % at d = 128 and S = 4096 against the pipelined form, whose packing the compiler places by itself.
   constexpr bool kSplitSoftmax = true;
-  auto pin_scores = [&](v16i (&acc)[kKeyTiles]) {
+  auto pin_scores = [&](v16i (&acc)[kKeyTiles]) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = 0; t < kKeyTiles; ++t) asm volatile("" : "+v"(acc[t]));
     asm volatile("" : "+v"(l_blk), "+v"(m_blk));
@@ -857,7 +890,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   constexpr bool kLoadsInMfmaPhase = true;
 #endif
   static_assert(!kLoadsInMfmaPhase || 2 * kRegionsPerWave <= kDSteps, "one tile load per output tile of GEMM 2");
-  auto phase_gemm2_merge = [&](int kb, const v4i (&pk)[kKeyTiles], int k_next, int v_next) {
+  auto phase_gemm2_merge = [&](int kb, const v4i (&pk)[kKeyTiles], int k_next, int v_next) __attribute__((always_inline)) {
 #ifdef FMHA_KO_MFMA
     if (kLoadsInMfmaPhase) {
       issue_k(k_next);
@@ -885,7 +918,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     if (FASTACC) t_run += take;
     float neg_take = FULLP ? take : -take;  // P carries the sign: P = -128 p (inc/fmha_i8.cuh:298); FULLP: P = 255 p
     asm volatile("" : "+v"(neg_take));  // a plain register operand: as a source modifier it would force the 64-bit encoding
-    auto merge_piece = [&](const v16i& oa, int u, int j) {  // four of the sixteen elements of output tile u
+    auto merge_piece = [&](const v16i& oa, int u, int j) __attribute__((always_inline)) {  // four of the sixteen elements of output tile u
 #pragma unroll
       for (int r = 4 * j; r < 4 * j + 4; ++r)
         o_f[u][r] = __builtin_fmaf(neg_take, FASTACC ? __int_as_float(oa[r]) : __int_as_float(oa[r]) - (FULLP ? kBaseFull : kBase),
@@ -900,7 +933,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     constexpr int kOaccBufs = FULLP ? 3 : 2;
     v16i oacc[kOaccBufs];
     auto ob = [&](int u) { return FULLP ? u % 3 : u & 1; };
-    auto read_start = [&](int u) {
+    auto read_start = [&](int u) __attribute__((always_inline)) {
       const int* cs = &lds_colsum[(kb & 1) * D + 32 * u + 4 * g];
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
@@ -909,7 +942,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         for (int bb = 0; bb < 4; ++bb) oacc[ob(u)][4 * a + bb] = w[bb];
       }
     };
-    auto read_tile = [&](int u) {
+    auto read_tile = [&](int u) __attribute__((always_inline)) {
 #ifdef FMHA_KO_LDS_READS
 #pragma unroll
       for (int t = 0; t < kKeyTiles; ++t) {
@@ -958,7 +991,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // reads of GEMM 2 hand lane (i32, g) sixteen keys of column 32u + i32 per key tile; v_dot4 against four ones sums
   // them, the two halves of the wavefront add up to the whole tile.  Rows of a tile that stand for keys which do not
   // exist (a ragged end) are counted like any other: their P is 0, i.e. the byte -128, and the two cancel.
-  auto phase_colsum = [&](int kb) {
+  auto phase_colsum = [&](int kb) __attribute__((always_inline)) {
     if (colsum_tile >= 0 && colsum_tile < kDSteps) {
       const int8_t* lds_v = &lds[kb & (kStages - 1)][1][0];
       typedef v2i __attribute__((address_space(3))) * lds_v2i_ptr;
@@ -1007,7 +1040,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // last block is replaced by the last block, which is then fetched again into the stage it already occupies (the
   // same bytes: harmless for the wavefronts reading it).  That keeps the wait counts below compile-time constants and
   // the key loop free of the compares and branches that a count depending on the position would need.
-  auto issue_first = [&]() {          // after barrier 0
+  auto issue_first = [&]() __attribute__((always_inline)) {          // after barrier 0
     if (n > 0) {
       if (FULLP && kOneBarrier) {  // in pairs, so that "all but the newest two tiles" means the same at every barrier
         issue_k(min(1, last));
@@ -1021,7 +1054,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       }
     }
   };
-  auto issue_for = [&](int i) {  // where GEMM 2 of block i is skipped
+  auto issue_for = [&](int i) __attribute__((always_inline)) {  // where GEMM 2 of block i is skipped
     issue_k(min(i + 3, last));
     issue_v(min(i + kVAhead, last));
   };
@@ -1090,10 +1123,14 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   int mx[2];
   // Where GEMM 1 is skipped the old scores are dead; saying so (an empty definition) keeps 64 registers from being
   // carried through the following MFMA phase.
-  auto forget_scores = [&]() {
+  auto forget_scores = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int t = 0; t < kKeyTiles; ++t) asm volatile("" : "=v"(acc[t]));
     asm volatile("" : "=v"(mx[0]), "=v"(mx[1]));
+  };
+  auto gemm1_of = [&](int kb) __attribute__((always_inline)) {  // GEMM 1 of block 0, which may or may not have masked keys
+    if (cls_of(kb) != 0) phase_gemm1(kb, acc, mx, true);
+    else phase_gemm1(kb, acc, mx, false);
   };
   // The wavefront in its MFMA phase gets the issue slots it asks for: an MFMA, an operand read or a merge instruction
   // that waits behind the other wavefront's softmax stream leaves the MFMA pipe idle, the reverse costs nothing.
@@ -1102,36 +1139,52 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   if (wave < kClassWaves) {
     prologue_waves_0_to_3();
     first_barrier();
-    if (n > 0 && works(0)) phase_gemm1(0, acc, mx);
+    if (n > 0 && works(0)) gemm1_of(0);
     else forget_scores();
     issue_first();
     int i = 0;
     // Steady state, as long as blocks i and i+1 exist and have no masked key: the same phases as the general loop
     // below with every decision taken (scalar compares and branches are not free: they stand in the issue stream of
-    // the wavefront that the barrier is waiting for).
+    // the wavefront that the barrier is waiting for).  A second loop of the same shape serves blocks with masked keys:
+    // what it adds is the reference's sentinel in the softmax and the GEMM 1 that starts masked keys at "gone" (for
+    // every block from the first one with a masked key on, whether the block has one or not: a branch between the
+    // two forms of GEMM 1 inside the loop makes the d = 128 kernel spill).  Blocks whose keys are all masked, and the
+    // last block, are left to the general loop.
+    auto steady_a = [&](int i, int cls, bool next_masked) __attribute__((always_inline)) {
+      v4i pk[kKeyTiles];
+      wait_v_for_colsum_a();
+      barrier_odd();
+      phase_softmax(i, cls, acc, pk, mx, kSplitSoftmax);
+      if (kSplitSoftmax) pin_scores(acc);
+      issue_after_softmax_a(i);
+      staged_writes_done();
+      wait_tiles(true);
+      barrier();
+      if (kStaged) staged_step(i);
+      else issue_after_barrier_a(i);
+      raise_priority();
+      if (kSplitSoftmax) {
+        pin_scores(acc);
+        phase_pack(acc, pk);
+      }
+      phase_gemm2_merge(i, pk, min(i + 3, last), min(i + kVAhead, last));
+      if (next_masked) phase_gemm1(i + 1, acc, mx, true);
+      else phase_gemm1(i + 1, acc, mx, false);
+      drop_priority();
+    };
     if (active) {
       align_loop();
       asm volatile(".rept %0\n\ts_nop 0\n\t.endr" :: "n"(kLoopPadA) : "memory");
-      for (; i + 1 < n && i + 1 < kb_plain; ++i) {
-        v4i pk[kKeyTiles];
-        wait_v_for_colsum_a();
-        barrier_odd();
-        phase_softmax(i, 0, acc, pk, mx, kSplitSoftmax);
-        if (kSplitSoftmax) pin_scores(acc);
-        issue_after_softmax_a(i);
-        staged_writes_done();
-        wait_tiles(true);
-        barrier();
-        if (kStaged) staged_step(i);
-        else issue_after_barrier_a(i);
-        raise_priority();
-        if (kSplitSoftmax) {
-          pin_scores(acc);
-          phase_pack(acc, pk);
+      for (; i + 1 < n && i + 1 < kb_plain; ++i) steady_a(i, 0, false);
+      if (!kStaged) {
+        int cls = i < n ? cls_of(i) : 2;
+        while (i + 1 < n && !(cls & 2)) {
+          const int cls_next = cls_of(i + 1);
+          if (cls_next & 2) break;
+          steady_a(i, cls, true);
+          cls = cls_next;
+          ++i;
         }
-        phase_gemm2_merge(i, pk, min(i + 3, last), min(i + kVAhead, last));
-        phase_gemm1(i + 1, acc, mx);
-        drop_priority();
       }
       if (kStaged) {
         staged_write();
@@ -1152,7 +1205,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       raise_priority();
       if (work) phase_gemm2_merge(i, pk, min(i + 3, last), min(i + kVAhead, last));
       else issue_in_mfma_phase(i);
-      if (i + 1 < n && works(i + 1)) phase_gemm1(i + 1, acc, mx);
+      if (i + 1 < n && works(i + 1)) phase_gemm1(i + 1, acc, mx, true);
       else forget_scores();
       drop_priority();
     }
@@ -1165,33 +1218,45 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     if (FULLP && !kOneBarrier) wait_all_but(3);  // V(0) has landed: K1 K2 V1 may be in flight
     barrier_odd();                             // barrier 1
     if (FULLP && n > 0) phase_colsum(0);
-    if (n > 0 && works(0)) phase_gemm1(0, acc, mx);
+    if (n > 0 && works(0)) gemm1_of(0);
     else forget_scores();
     if (FULLP) colsum_written();
     int i = 0;
-    if (active) {  // steady state, see above
+    auto steady_b = [&](int i, int cls, bool next_masked) __attribute__((always_inline)) {  // see steady_a above
+      v4i pk[kKeyTiles];
+      wait_tiles(false);
+      barrier();
+      phase_softmax(i, cls, acc, pk, mx, kSplitSoftmax);
+      if (kSplitSoftmax) pin_scores(acc);
+      if (kStaged) staged_step(i);
+      else issue_after_softmax(i);
+      wait_v_for_colsum_b();
+      barrier_odd();
+      raise_priority();
+      if (kSplitSoftmax) {
+        pin_scores(acc);
+        phase_pack(acc, pk);
+      }
+      phase_gemm2_merge(i, pk, min(i + 3, last), min(i + kVAhead, last));
+      if (FULLP) phase_colsum(i + 1);
+      if (next_masked) phase_gemm1(i + 1, acc, mx, true);
+      else phase_gemm1(i + 1, acc, mx, false);
+      if (FULLP) colsum_written();
+      drop_priority();
+      staged_writes_done();
+    };
+    if (active) {
       align_loop();
-      for (; i + 1 < n && i + 1 < kb_plain; ++i) {
-        v4i pk[kKeyTiles];
-        wait_tiles(false);
-        barrier();
-        phase_softmax(i, 0, acc, pk, mx, kSplitSoftmax);
-        if (kSplitSoftmax) pin_scores(acc);
-        if (kStaged) staged_step(i);
-        else issue_after_softmax(i);
-        wait_v_for_colsum_b();
-        barrier_odd();
-        raise_priority();
-        if (kSplitSoftmax) {
-          pin_scores(acc);
-          phase_pack(acc, pk);
+      for (; i + 1 < n && i + 1 < kb_plain; ++i) steady_b(i, 0, false);
+      if (!kStaged) {
+        int cls = i < n ? cls_of(i) : 2;
+        while (i + 1 < n && !(cls & 2)) {
+          const int cls_next = cls_of(i + 1);
+          if (cls_next & 2) break;
+          steady_b(i, cls, true);
+          cls = cls_next;
+          ++i;
         }
-        phase_gemm2_merge(i, pk, min(i + 3, last), min(i + kVAhead, last));
-        if (FULLP) phase_colsum(i + 1);
-        phase_gemm1(i + 1, acc, mx);
-        if (FULLP) colsum_written();
-        drop_priority();
-        staged_writes_done();
       }
       if (kStaged) {
         staged_write();
@@ -1212,7 +1277,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       if (work) phase_gemm2_merge(i, pk, min(i + 3, last), min(i + kVAhead, last));
       else issue_in_mfma_phase(i);
       if (FULLP && i + 1 < n) phase_colsum(i + 1);
-      if (i + 1 < n && works(i + 1)) phase_gemm1(i + 1, acc, mx);
+      if (i + 1 < n && works(i + 1)) phase_gemm1(i + 1, acc, mx, true);
       else forget_scores();
       if (FULLP) colsum_written();
       drop_priority();
