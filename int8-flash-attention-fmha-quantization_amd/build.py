@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 LIB_PATH = os.path.join(HERE, "libfmha_i8.so")
 SOURCES = [os.path.join(HERE, "csrc", "fmha_i8_api.hip"), os.path.join(HERE, "csrc", "fmha_quant.hip")]
-DEPENDS = SOURCES + [os.path.join(HERE, "csrc", "fmha_i8_kernel.hip"),
+DEPENDS = SOURCES + [os.path.join(HERE, "csrc", "fmha_i8_kernel.hip"), os.path.join(HERE, "csrc", "fmha_i8_test_builds.h"),
                      os.path.join(ROOT, "include", "fmha_i8.h"), os.path.join(ROOT, "include", "fmha_param_i8.h"),
                      os.path.join(ROOT, "include", "fmha_quant.h")]
 # Packed-FP32 instruction selection is switched off for all device code (a flag for hipcc's device pass; the host pass

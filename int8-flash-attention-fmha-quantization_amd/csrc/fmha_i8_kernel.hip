@@ -70,44 +70,14 @@ constexpr float kLog2PscaleFull = -7.00560236f;  // log2(255 / 32767)
 constexpr int kBaseBitsFull = 0x3E400000;
 constexpr float kBaseFull = __builtin_bit_cast(float, kBaseBitsFull);
 
-// FMHA_CHECK_BOUNDS (a test build, never the shipped library): every global access of the kernel is first checked
-// against the tensor - for K and V the head - it belongs to; an access that would leave it is counted in
-// g_fmha_oob_count and redirected to the first byte, so that the run ends normally and the test can read the count.
-// An out-of-bounds READ changes no result and, inside a caching allocator's pool, raises no fault: nothing else shows it.
-#ifdef FMHA_CHECK_BOUNDS
-__device__ int g_fmha_oob_count;
-__device__ __forceinline__ bool fmha_in_bounds(bool ok) {
-  if (!ok) atomicAdd(&g_fmha_oob_count, 1);
-  return ok;
-}
-#else
-__device__ __forceinline__ constexpr bool fmha_in_bounds(bool) { return true; }
-#endif
+}  // namespace fmha_i8_gfx950
 
-// Further test builds (tests/Makefile, target `variants`; never the shipped library).  They exist so that every claim
-// about where the time goes can be re-measured: each one removes or changes ONE thing and is timed and counted
-// against the shipped kernel.  The knock-outs produce garbage results on purpose.
-//   FMHA_KO_SOFTMAX      the block softmax is not computed (P, block maximum and row sum are left undefined)
-//   FMHA_KO_MFMA         GEMM 2 + merge and GEMM 1 + row maximum are not computed (with FMHA_KO_SOFTMAX: the key loop
-//                        is tile loads, waits and barriers only)
-//   FMHA_KO_SCALE_RUN, FMHA_KO_EXP_RUN, FMHA_KO_SUM_RUN   one of the three dense runs of the steady-state softmax is
-//                        left out: the 64 scale fmas (and conversions), the 64 exponentials, the 64 + 4 row-sum adds
-//   FMHA_KO_LDS_READS    the MFMA operands are undefined registers instead of LDS reads
-//   FMHA_KO_TILE_LOADS   no K/V tile is fetched after the prologue
-//   FMHA_NO_SWIZZLE      K and V tiles lie in LDS as plain [key][d] rows (results unchanged, bank conflicts are not)
-//   FMHA_OLD_K_SWIZZLE   the K swizzle this kernel had first, which leaves a two-way conflict on every K operand read
-//   FMHA_TRACE_TICKS     every wavefront records the shader-clock time of each barrier arrival and departure
-//   FMHA_VGPR_STAGED_LOADS  the "before" of the direct-to-LDS tile loads: in the steady-state loop at d = 128 a K/V tile
-//                        goes HBM -> registers (global_load_dwordx4) and, one key block later, registers -> LDS
-//                        (ds_write_b128), the way a kernel without LDS-DMA has to do it; same bytes in the same places
-//   FMHA_TWO_BARRIERS    the "before" of the one-barrier schedule: a second workgroup barrier per key block, between the
-//                        two phases (results unchanged)
-#ifdef FMHA_TRACE_TICKS
-// [workgroup][wavefront][64]: lane n < 62 of one register holds the n-th time stamp (s_memtime, shader clock), lanes 62
-// and 63 the 100 MHz counter at the start and the end of the wavefront; written out when the wavefront ends.
-constexpr int kTraceWorkgroups = 4096;
-__device__ unsigned g_fmha_trace[kTraceWorkgroups * 8 * 64];
-#endif
+// Test builds (knock-outs, "before" layouts and schedules, time stamps, bounds checks): compile-time flags, all false
+// in the shipped library, and the few helpers they need.  `fmha_in_bounds` comes from there too: it is the constant
+// `true` unless the build checks every global access.
+#include "fmha_i8_test_builds.h"
+
+namespace fmha_i8_gfx950 {
 
 struct KernelArgs {
   const int8_t* q;
@@ -130,25 +100,17 @@ struct KernelArgs {
 // whose 16-lane groups touch keys {0,1,2,3,8,9,10,11} (+4, +16, +20) of a 32-key slab.
 template <int D>
 __device__ __forceinline__ int k_swizzle(int row) {
-#ifdef FMHA_NO_SWIZZLE
-  return 0;
-#else
+  if constexpr (test_build::kNoSwizzle) return 0;
+  // (the swizzle this kernel had first: rows r and r+8 / r+4 collide, a two-way conflict)
+  if constexpr (test_build::kOldKSwizzle) return D == 128 ? (row & 7) : ((row >> 1) & 3);
   // Sixteen lanes are served per cycle: rows r .. r+15 of one 16-byte chunk column.  A row is D bytes, the banks repeat
   // every 256 bytes, so rows 256/D apart start in the same bank: those rows must get different chunks.
-#ifdef FMHA_OLD_K_SWIZZLE
-  return D == 128 ? (row & 7) : ((row >> 1) & 3);   // (two-way conflicts: rows r and r+8 / r+4 collide)
-#else
   return D == 128 ? ((row >> 1) & 7) : ((row >> 2) & 3);
-#endif
-#endif
 }
 template <int D>
 __device__ __forceinline__ int v_swizzle(int key) {
-#ifdef FMHA_NO_SWIZZLE
-  return 0;
-#else
+  if constexpr (test_build::kNoSwizzle) return 0;
   return D == 128 ? ((key & 3) | ((key >> 1) & 4)) : (((key >> 1) & 1) | ((key >> 2) & 2));
-#endif
 }
 
 // P packing: four floats y_i in [-1, 1] -> four int8 bytes rne(32767 * y_i).  v_cvt_pknorm_i16_f32 converts two at a
@@ -290,11 +252,9 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(dst), "v"(src), "s"(gbase) : "memory");
   };
-  bool prologue_done = false;  // (FMHA_KO_TILE_LOADS)
+  bool prologue_done = false;  // (the test build without tile loads still fetches the tiles of the prologue)
   auto issue_region = [&](const int8_t* gbase, int kb, int which, int goff, int it) __attribute__((always_inline)) {  // which: 0 = K, 1 = V
-#ifdef FMHA_KO_TILE_LOADS
-    if (prologue_done) return;
-#endif
+    if (test_build::kNoTileLoads && prologue_done) return;
     const int region = (it * kWaves + wave) % kRegions;
     if (RAGGED && short_seq) {
       issue_short_region(gbase, which, goff, region);
@@ -366,42 +326,36 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // GEMM 1 - start at 8-byte-aligned addresses (fast) or straddle two (slow).  The right distance is found by timing
   // (tests/variant_timing.py, -DFMHA_LOOP_PAD_A=0 against 1) whenever the code between the boundary and the loop changes.
   auto align_loop = [&]() { asm volatile(".p2align 6" ::: "memory"); };
-#ifdef FMHA_LOOP_PAD_A
-  constexpr int kLoopPadA = FMHA_LOOP_PAD_A;
-#else
-  constexpr int kLoopPadA = D == 64 ? 1 : 0;  // s_nops between the boundary and the loop of wavefronts 0..3 (see above)
-#endif
-#ifdef FMHA_TRACE_TICKS
+  // s_nops between the boundary and the loop of wavefronts 0..3 (see above)
+  constexpr int kLoopPadA = test_build::kLoopPadA >= 0 ? test_build::kLoopPadA : (D == 64 ? 1 : 0);
+  // (test build with time stamps: every wavefront records the shader clock at each barrier arrival and departure, in the
+  // lanes of one register; lanes 62 and 63 take the constant-rate 100 MHz counter when the wavefront starts and ends,
+  // which with the first and the last stamp gives the shader clock the kernel actually ran at)
   unsigned trace_reg = 0;
   int trace_n = 0;
   auto stamp = [&]() {
-    unsigned long long t;
-    asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t) :: "memory");
-    if (trace_n < 62)
-      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tv_writelane_b32 %0, %1, m0" : "+v"(trace_reg) : "s"((unsigned)t), "s"(__builtin_amdgcn_readfirstlane(trace_n)));
-    ++trace_n;
+    if constexpr (test_build::kTraceTicks) {
+      unsigned long long t;
+      asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t) :: "memory");
+      if (trace_n < 62)
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tv_writelane_b32 %0, %1, m0" : "+v"(trace_reg) : "s"((unsigned)t), "s"(__builtin_amdgcn_readfirstlane(trace_n)));
+      ++trace_n;
+    }
+  };
+  auto stamp_real = [&](int slot) {
+    if constexpr (test_build::kTraceTicks) {
+      unsigned long long t;
+      asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t) :: "memory");
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tv_writelane_b32 %0, %1, m0" : "+v"(trace_reg) : "s"((unsigned)t), "s"(slot));
+    }
   };
   stamp();
-  // lanes 62 and 63: the constant-rate counter (100 MHz) when the wavefront starts and ends; with the first and the last
-  // s_memtime stamp it gives the shader clock the kernel actually ran at
-  auto stamp_real = [&](int slot) {
-    unsigned long long t;
-    asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t) :: "memory");
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tv_writelane_b32 %0, %1, m0" : "+v"(trace_reg) : "s"((unsigned)t), "s"(slot));
-  };
   stamp_real(62);
   auto barrier = [&]() { stamp(); asm volatile("s_barrier" ::: "memory"); stamp(); };
-#else
-  auto barrier = [&]() { asm volatile("s_barrier" ::: "memory"); };
-#endif
 
   // One workgroup barrier per key block, or (a test build) two: see the schedule below.
   // (FULLP at d = 64 keeps two: with one it measures 10 % slower, at d = 128 4 to 7 % faster.)
-#ifdef FMHA_TWO_BARRIERS
-  constexpr bool kOneBarrier = false;
-#else
-  constexpr bool kOneBarrier = !(FULLP && D == 64);
-#endif
+  constexpr bool kOneBarrier = !test_build::kTwoBarriers && !(FULLP && D == 64);
   constexpr int kVAhead = (FULLP && kOneBarrier) ? 3 : 2;
 
   const int row0 = qb * kBlockQ + wave * 32;  // first query row of this wavefront
@@ -627,20 +581,22 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // 8a+4+bb, so the scalar unit builds them from the block's mask bits - written into the accumulator registers
   // themselves, tile by tile, in front of the tile's MFMAs.
   auto phase_gemm1 = [&](int kb, v16i (&acc)[kKeyTiles], int (&mx)[2], bool masked = false) __attribute__((always_inline)) {
-#ifdef FMHA_KO_MFMA
+    if constexpr (test_build::kNoMfma) {
 #pragma unroll
-    for (int t = 0; t < kKeyTiles; ++t) asm volatile("" : "=v"(acc[t]));
-    asm volatile("" : "=v"(mx[0]), "=v"(mx[1]));
-    return;
-#endif
+      for (int t = 0; t < kKeyTiles; ++t) test_build::undefined(acc[t]);
+      test_build::undefined(mx[0]);
+      test_build::undefined(mx[1]);
+      return;
+    }
     const int8_t* lds_k = &lds[kb & (kStages - 1)][0][0];
     const v16i zero_c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     v4i ka[2][kDSteps];  // operand reads run one key tile ahead of the MFMAs that consume them
-#ifdef FMHA_KO_LDS_READS
-    auto read_k = [&](int) { v4i undefined; asm volatile("" : "=v"(undefined)); return undefined; };
-#else
-    auto read_k = [&](int off) { return *reinterpret_cast<const v4i*>(lds_k + off); };
-#endif
+    auto read_k = [&](int off) {
+      v4i operand;
+      if constexpr (test_build::kNoLdsReads) test_build::undefined(operand);
+      else operand = *reinterpret_cast<const v4i*>(lds_k + off);
+      return operand;
+    };
     unsigned mw[kKeyTiles];  // masked: the block's mask bits, bit j of word t <-> key 32 t + j of the block
     int gone = BIAS ? (int)0xFF000000 : -(1 << 30);
     if (masked) {
@@ -719,14 +675,15 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // steady-state loop): everything but the P packing, in three dense runs - 64 scale fmas, 64 exponentials, 64 + 4 adds -
   // and the exponentials are left in acc (as float bits) for phase_pack, which runs at the head of the MFMA phase.
   auto phase_softmax = [&](int kb, int cls, v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles], int (&mx)[2], bool split = false) __attribute__((always_inline)) {
-#ifdef FMHA_KO_SOFTMAX
-    if (!split) {
+    if constexpr (test_build::kNoSoftmax) {
+      if (!split) {
 #pragma unroll
-      for (int t = 0; t < kKeyTiles; ++t) asm volatile("" : "=v"(pk[t]));
+        for (int t = 0; t < kKeyTiles; ++t) test_build::undefined(pk[t]);
+      }
+      test_build::undefined(m_blk);
+      test_build::undefined(l_blk);
+      return;
     }
-    asm volatile("" : "=v"(m_blk), "=v"(l_blk));
-    return;
-#endif
     auto sf = [&](int t, int r) -> float { return BIAS ? __int_as_float(acc[t][r]) : (float)acc[t][r]; };
     l_blk = 0.f;
     // (cls != 0: some keys of this block are masked out.  GEMM 1 has seen to it that their scores lose every maximum
@@ -764,33 +721,59 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
 #pragma unroll
         for (int qd = 0; qd < kQuads; ++qd)
 #pragma unroll
-#ifdef FMHA_KO_SCALE_RUN
-          for (int j = 0; j < 4; ++j) xs[qd][j] = __int_as_float(acc[qd / 4][4 * (qd % 4) + j]);
-#else
-          for (int j = 0; j < 4; ++j) xs[qd][j] = __builtin_fmaf(sf(qd / 4, 4 * (qd % 4) + j), c2, -offq);
-#endif
+          for (int j = 0; j < 4; ++j)
+            xs[qd][j] = test_build::kNoScaleRun ? __int_as_float(acc[qd / 4][4 * (qd % 4) + j])
+                                                : __builtin_fmaf(sf(qd / 4, 4 * (qd % 4) + j), c2, -offq);
 #pragma unroll
         for (int qd = 0; qd < kQuads; ++qd) asm volatile("" : "+v"(xs[qd][0]), "+v"(xs[qd][1]), "+v"(xs[qd][2]), "+v"(xs[qd][3]));
         __builtin_amdgcn_sched_barrier(0);
-#ifndef FMHA_KO_EXP_RUN
+        if constexpr (!test_build::kNoExpRun) {
 #pragma unroll
-        for (int qd = 0; qd < kQuads; ++qd)
+          for (int qd = 0; qd < kQuads; ++qd)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) xs[qd][j] = __builtin_amdgcn_exp2f(xs[qd][j]);
-#endif
+            for (int j = 0; j < 4; ++j) xs[qd][j] = __builtin_amdgcn_exp2f(xs[qd][j]);
+        }
 #pragma unroll
         for (int qd = 0; qd < kQuads; ++qd) asm volatile("" : "+v"(xs[qd][0]), "+v"(xs[qd][1]), "+v"(xs[qd][2]), "+v"(xs[qd][3]));
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (test_build::kMfmaRowSum) {
+          // (test build: the row sum on the matrix pipe.  The exponentials are rounded to half precision two at a time
+          // and eight of them per lane go into one v_mfma_f32_16x16x32_f16 as the B operand - lane l brings eight keys
+          // of query l%32, so column n of B holds query n in the k-slots of lanes n and n+32 and query n+16 in those of
+          // lanes n+16 and n+48 - against an A operand whose rows 0..3 and 8..11 are 1 on the first kind of k-slot and 0
+          // on the second, rows 4..7 and 12..15 the other way round: every lane then receives, four times, the sum over
+          // both lanes of its own query.  32 conversions and 8 MFMAs in place of 67 additions and the lane exchange.)
+          typedef float f2 __attribute__((ext_vector_type(2)));
+          typedef float f4 __attribute__((ext_vector_type(4)));
+          typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+          typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+          const _Float16 one = ((((lane & 15) >> 2) ^ (lane >> 4)) & 1) ? (_Float16)0.f : (_Float16)1.f;
+          const h8 ones = {one, one, one, one, one, one, one, one};
+          f4 lsum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int qd = 0; qd < kQuads; qd += 2) {
+            const h2 p0 = __builtin_convertvector(f2{xs[qd][0], xs[qd][1]}, h2), p1 = __builtin_convertvector(f2{xs[qd][2], xs[qd][3]}, h2);
+            const h2 p2 = __builtin_convertvector(f2{xs[qd + 1][0], xs[qd + 1][1]}, h2), p3 = __builtin_convertvector(f2{xs[qd + 1][2], xs[qd + 1][3]}, h2);
+            const h8 b = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+            lsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, b, lsum, 0, 0, 0);
+          }
+#pragma unroll
+          for (int qd = 0; qd < kQuads; ++qd)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[qd / 4][4 * (qd % 4) + j] = __float_as_int(xs[qd][j]);
+          l_blk = lsum[0];
+          return;
+        }
 #pragma unroll
         for (int qd = 0; qd < kQuads; ++qd) {
-#ifdef FMHA_KO_SUM_RUN
-          if (qd == 0) l_blk += xs[0][0];
-#else
-          float s01 = xs[qd][0] + xs[qd][1];
-          const float s23 = xs[qd][2] + xs[qd][3];
-          s01 += s23;
-          l_blk += s01;
-#endif
+          if constexpr (test_build::kNoSumRun) {
+            if (qd == 0) l_blk += xs[0][0];
+          } else {
+            float s01 = xs[qd][0] + xs[qd][1];
+            const float s23 = xs[qd][2] + xs[qd][3];
+            s01 += s23;
+            l_blk += s01;
+          }
 #pragma unroll
           for (int j = 0; j < 4; ++j) acc[qd / 4][4 * (qd % 4) + j] = __float_as_int(xs[qd][j]);
         }
@@ -846,11 +829,11 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   };
   // P packing of the exponentials that phase_softmax(split) left in acc: P^T as the B operand of GEMM 2.
   auto phase_pack = [&](v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles]) __attribute__((always_inline)) {
-#ifdef FMHA_KO_SOFTMAX
+    if constexpr (test_build::kNoSoftmax) {
 #pragma unroll
-    for (int t = 0; t < kKeyTiles; ++t) asm volatile("" : "=v"(pk[t]));
-    return;
-#endif
+      for (int t = 0; t < kKeyTiles; ++t) test_build::undefined(pk[t]);
+      return;
+    }
     align8();
 #pragma unroll
     for (int qd = 0; qd < 4 * kKeyTiles; ++qd) {
@@ -884,24 +867,20 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // waits of the MFMA chain (-7 % at d = 64 against issuing them after the softmax, -0.6 % at d = 128 against issuing them
   // in front of the MFMA phase).  The other placements are kept for the test build that stages the tiles through
   // registers, which needs the loads of a key block in one place.
-#ifdef FMHA_VGPR_STAGED_LOADS
-  constexpr bool kLoadsInMfmaPhase = D == 64;
-#else
-  constexpr bool kLoadsInMfmaPhase = true;
-#endif
+  constexpr bool kLoadsInMfmaPhase = !test_build::kStagedLoads || D == 64;
   static_assert(!kLoadsInMfmaPhase || 2 * kRegionsPerWave <= kDSteps, "one tile load per output tile of GEMM 2");
   auto phase_gemm2_merge = [&](int kb, const v4i (&pk)[kKeyTiles], int k_next, int v_next) __attribute__((always_inline)) {
-#ifdef FMHA_KO_MFMA
-    if (kLoadsInMfmaPhase) {
-      issue_k(k_next);
-      issue_v(v_next);
-    }
-    // (the softmax that produced these stays: an empty statement that reads them)
+    if constexpr (test_build::kNoMfma) {
+      if (kLoadsInMfmaPhase) {
+        issue_k(k_next);
+        issue_v(v_next);
+      }
 #pragma unroll
-    for (int t = 0; t < kKeyTiles; ++t) asm volatile("" :: "v"(pk[t]));
-    asm volatile("" :: "v"(m_blk), "v"(l_blk));
-    return;
-#endif
+      for (int t = 0; t < kKeyTiles; ++t) test_build::consume(pk[t]);  // (the softmax that produced these stays)
+      test_build::consume(m_blk);
+      test_build::consume(l_blk);
+      return;
+    }
     if (__ballot(m_blk > m_ref + kLazyLog2) != 0) {
       const float m_new = fmaxf(m_ref, m_blk);
       const float keep = __builtin_amdgcn_exp2f(m_ref - m_new);
@@ -943,14 +922,14 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       }
     };
     auto read_tile = [&](int u) __attribute__((always_inline)) {
-#ifdef FMHA_KO_LDS_READS
+      if constexpr (test_build::kNoLdsReads) {
 #pragma unroll
-      for (int t = 0; t < kKeyTiles; ++t) {
-        asm volatile("" : "=v"(va[u & 1][t][0]));
-        asm volatile("" : "=v"(va[u & 1][t][1]));
+        for (int t = 0; t < kKeyTiles; ++t) {
+          test_build::undefined(va[u & 1][t][0]);
+          test_build::undefined(va[u & 1][t][1]);
+        }
+        return;
       }
-      return;
-#endif
 #pragma unroll
       for (int t = 0; t < kKeyTiles; ++t) {
         va[u & 1][t][0] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(lds_v + v_read_off[u] + 32 * t * D));
@@ -1069,50 +1048,11 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // barrier that follows it
   auto issue_after_softmax_a = [&](int i) { if (!kOneBarrier) issue_after_softmax(i); };
   auto issue_after_barrier_a = [&](int i) { if (kOneBarrier) issue_after_softmax(i); };
-#ifdef FMHA_VGPR_STAGED_LOADS
-  // One pair of tiles (K(i+3), V(i+2)) on its way through this wavefront's registers: loaded at the issue point of
-  // key block i, written to LDS at the issue point of key block i+1 - still a whole key block before the barrier that
-  // publishes it.  Only where the tiles would otherwise be requested in front of the MFMA phase (d = 128).
-  constexpr bool kStaged = kOneBarrier && !kLoadsInMfmaPhase && !RAGGED;
-  v4i staged[2][kRegionsPerWave];
-  int staged_kb[2] = {0, 0};
-  bool have_staged = false;
-  auto staged_write = [&]() {
-    if (!have_staged) return;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#pragma unroll
-    for (int which = 0; which < 2; ++which)
-#pragma unroll
-      for (int it = 0; it < kRegionsPerWave; ++it) {
-        asm volatile("" : "+v"(staged[which][it]));
-        const int region = (it * kWaves + wave) % kRegions;
-        *reinterpret_cast<v4i*>(&lds[staged_kb[which] & (kStages - 1)][which][region * 1024 + 16 * lane]) = staged[which][it];
-      }
-    have_staged = false;
-  };
-  auto staged_step = [&](int i) {
-    staged_write();
-    staged_kb[0] = min(i + 3, last);
-    staged_kb[1] = min(i + 2, last);
-#pragma unroll
-    for (int which = 0; which < 2; ++which)
-#pragma unroll
-      for (int it = 0; it < kRegionsPerWave; ++it) {
-        const int8_t* gp = (which ? vg : kg) + (long)staged_kb[which] * kTileBytes;
-        const int region = (it * kWaves + wave) % kRegions;
-        const int src = (which ? ld_goff_v : ld_goff_k) + region * 1024;
-        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(staged[which][it]) : "v"(src), "s"(gp) : "memory");
-      }
-    have_staged = true;
-  };
-  // LDS writes are not waited for by the hand-written barrier
-  auto staged_writes_done = [&]() { if (kStaged) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
-#else
-  constexpr bool kStaged = false;
-  auto staged_write = [&]() {};
-  auto staged_step = [&](int) {};
-  auto staged_writes_done = [&]() {};
-#endif
+  // (test build that stages the tiles of the steady-state loop through registers, the "before" of the direct-to-LDS
+  // loads: staged_step(i) loads the pair of tiles of issue point i into registers and writes the pair of issue point
+  // i-1 to LDS.  The definitions live with the other test builds; in the shipped library kStaged is false and the three
+  // calls are empty.)
+  FMHA_STAGED_LOAD_LAMBDAS
   // FULLP with two barriers per key block: V(m) is summed by wavefronts 4..7 in tick 2m+1, one tick before its GEMM 2,
   // so it is barrier 2m+1 that publishes it.  Wavefronts 0..3 arrive there from their MFMA phase (the pair issued last may stay in flight),
   // wavefronts 4..7 from their softmax (the pair they have just issued; none where the loads go out in the MFMA phase).
@@ -1284,11 +1224,9 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     }
   }
   wait_all();  // nothing may still be writing LDS when the wavefront ends (only possible when every key is masked)
-#ifdef FMHA_TRACE_TICKS
   stamp();
   stamp_real(63);
-  if (blockIdx.x < kTraceWorkgroups) g_fmha_trace[(blockIdx.x * 8 + wave) * 64 + lane] = trace_reg;
-#endif
+  test_build::write_trace(blockIdx.x, wave, lane, trace_reg);
   if (!active) return;
 
   // ---- epilogue: normalise, requantise, store (inc/fmha_i8.cuh:318-332) --------------------------------------------
