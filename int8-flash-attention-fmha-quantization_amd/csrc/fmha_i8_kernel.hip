@@ -324,10 +324,11 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // one too; the loop of wavefronts 4..7 measures the same either way, and so do both loops at d = 128).  What flips
   // with those 4 bytes is whether the eight v_max3_i32 at the top of the loop - the first readers of the last MFMA of
   // GEMM 1 - start at 8-byte-aligned addresses (fast) or straddle two (slow).  The right distance is found by timing
-  // (tests/variant_timing.py, -DFMHA_LOOP_PAD_A=0 against 1) whenever the code between the boundary and the loop changes.
+  // (the test builds loop_pad_a0 and loop_pad_a1, -DFMHA_LOOP_PAD_A=0 against 1) whenever the code between the boundary
+  // and the loop changes; tests/test_gpu_variant_builds.py holds the shipped library to the faster of the two.
   auto align_loop = [&]() { asm volatile(".p2align 6" ::: "memory"); };
   // s_nops between the boundary and the loop of wavefronts 0..3 (see above)
-  constexpr int kLoopPadA = test_build::kLoopPadA >= 0 ? test_build::kLoopPadA : (D == 64 ? 1 : 0);
+  constexpr int kLoopPadA = test_build::kLoopPadA >= 0 ? test_build::kLoopPadA : 0;
   // (test build with time stamps: every wavefront records the shader clock at each barrier arrival and departure, in the
   // lanes of one register; lanes 62 and 63 take the constant-rate 100 MHz counter when the wavefront starts and ends,
   // which with the first and the last stamp gives the shader clock the kernel actually ran at)
@@ -368,6 +369,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   float m_ref;             // reference exponent of the running O and l (base-2 units)
   float t_run;             // FASTACC: sum of the merge weights, i.e. how much of kBase the running O carries
   float l_run;             // running row sum, in units of 1/128 (it sums 128*p)
+  bool merged_any = false; // some key block has been merged into O, l and t
   const float c2 = BIAS ? args.c2 * kBaseScale : args.c2;  // exponent per unit of sf() below
   const float bias_c2 = BIAS ? kBase * c2 : 0.f;
   float magic;
@@ -885,13 +887,16 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       const float m_new = fmaxf(m_ref, m_blk);
       const float keep = __builtin_amdgcn_exp2f(m_ref - m_new);
       m_ref = m_new;
-      l_run *= keep;
-      if (FASTACC) t_run *= keep;
+      if (merged_any) {  // (the first block always comes here, and has nothing to rescale: O, l and t are still 0)
+        l_run *= keep;
+        if (FASTACC) t_run *= keep;
 #pragma unroll
-      for (int u = 0; u < kDSteps; ++u)
+        for (int u = 0; u < kDSteps; ++u)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o_f[u][r] *= keep;
+          for (int r = 0; r < 16; ++r) o_f[u][r] *= keep;
+      }
     }
+    merged_any = true;
     const float take = __builtin_amdgcn_exp2f(m_blk - m_ref);
     l_run = __builtin_fmaf(take, l_blk, l_run);
     if (FASTACC) t_run += take;
