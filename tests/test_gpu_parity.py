@@ -261,6 +261,58 @@ def test_every_kernel_variant(pkg, orc, dev, S, d, qk_scale, vo_ratio):
     check(gpu_run(pkg, dev, c, **kw), want, "variant S=%d d=%d qk=%g vo=%g" % (S, d, qk_scale, vo_ratio))
 
 
+# Key blocks come in three kinds - no masked key (P), some (M), all (F) - and the kernel serves them with three loops
+# (a steady-state loop for runs of P, a second one from the first M on, a general loop for F blocks and the last
+# block); masked keys of an M block are handled where GEMM 1 starts its accumulators.  Every transition between the
+# loops, at both head sizes and both block sizes, full-range P included; a masked key also carries the largest score
+# of its row (K = Q there), so that a mask that is ignored cannot go unnoticed.
+BLOCK_PATTERNS = ["PMPF", "MPPM", "FPMP", "PPFM", "MMMM", "FFPF", "PFFM", "MFMP", "PPPM", "MPPP", "PMMPPFMP", "F", "M", "FM", "MF"]
+
+
+@pytest.mark.parametrize("d,block", [(128, 128), (64, 128), (128, 64), (64, 64)])
+@pytest.mark.parametrize("full_range_p", [False, True])
+def test_every_sequence_of_block_kinds(pkg, orc, dev, d, block, full_range_p):
+    import torch
+    rng = np.random.default_rng([d, block, int(full_range_p)])
+    for pattern in BLOCK_PATTERNS:
+        n = len(pattern)
+        S = n * block
+        pattern_here = pattern
+        if block == 64 and S % 128 == 0:  # (a multiple of 128 runs blocks of 128 keys: one more block of 64)
+            pattern_here, S = pattern + "P", S + 64
+        if block == 128 and S % 128 != 0:
+            continue
+        B, H = 2, 2
+        c = fc.make_inputs(B, H, S, d, dist="normal", sigma=1.0, pad="none", seed=int(rng.integers(1 << 30)))
+        mask = np.zeros((B, S), np.int8)
+        for b in range(B):
+            for i, kind in enumerate(pattern_here if b == 0 else pattern_here[::-1]):
+                lo = i * block
+                if kind == "F":
+                    mask[b, lo:lo + block] = 1
+                elif kind == "M":
+                    mask[b, lo:lo + block] = (rng.random(block) < 0.3).astype(np.int8)
+                    mask[b, lo + int(rng.integers(block))] = 0   # at least one key stays
+                    mask[b, lo + int(rng.integers(block))] = 3   # ... and one goes, with a byte other than 1
+        c["mask"] = mask
+        # masked keys that would win every maximum: K row = Q row of the same position, scaled up
+        kq = np.clip(c["q"].astype(np.int32) * 2, -127, 127).astype(np.int8)
+        for b in range(B):
+            gone = np.nonzero(mask[b])[0][::7]
+            c["k"][b][:, gone, :] = kq[b][:, gone, :]
+        q, k, v, m = to_dev(dev, c["q"], c["k"], c["v"], c["mask"])
+        o = pkg.fmha_infer_i8(q, k, v, m, c["q_amax"], c["k_amax"], c["v_amax"], c["o_amax"], full_range_p=full_range_p)
+        torch.cuda.synchronize()
+        blk = 128 if S % 128 == 0 else 64
+        if full_range_p:
+            want = orc.fmha_i8_blockwise_cross(c["q"], c["k"], c["v"], c["mask"], c["q_amax"], c["k_amax"], c["v_amax"],
+                                               c["o_amax"], block=blk, full_range_p=True)
+        else:
+            want = orc.fmha_i8_blockwise(c["q"], c["k"], c["v"], c["mask"], c["q_amax"], c["k_amax"], c["v_amax"],
+                                         c["o_amax"], block=blk)
+        check(o.cpu().numpy(), np.asarray(want).reshape(o.shape), "blocks %s d=%d block=%d full=%s" % (pattern_here, d, blk, full_range_p))
+
+
 @pytest.mark.parametrize("S,d", [(256, 128), (192, 64)])
 def test_zero_scale_with_masked_keys(pkg, orc, dev, S, d):
     """q_amax = 0 (an all-zero Q tensor quantised by abs-max): every score scales to 0, the softmax is uniform over the
