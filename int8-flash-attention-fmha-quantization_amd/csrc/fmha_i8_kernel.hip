@@ -24,12 +24,15 @@
 //     so that the MFMA pipe never waits for an issue slot.  One workgroup barrier per key block publishes the tiles;
 //   * the softmax is written for instruction count and issue order: exp in the base-2 domain with every scale folded
 //     into one fma, v_max3 on the raw accumulators for the row maximum, P converted two at a time by
-//     v_cvt_pknorm_i16_f32 and packed by v_perm_b32, the steady-state loop (blocks without masked keys) running the
-//     scale fmas, the exponentials and the sums as three dense runs with the P packing at the head of the MFMA phase,
-//     the general loop with every exponential followed by instructions that do not need the transcendental unit, the
+//     v_cvt_pknorm_i16_f32 and packed by v_perm_b32, the steady-state loops running the scale fmas, the exponentials
+//     and the sums as three dense runs with the P packing at the head of the MFMA phase, the general loop (the last
+//     block) with every exponential followed by instructions that do not need the transcendental unit, the
 //     int32 accumulators of both GEMMs started at the bit pattern of a float (an MFMA inline
 //     constant) so that they can be read as floats without a convert, the running O only rescaled when a row maximum
 //     jumps by more than 2^kLazyLog2, and O normalised once, in the epilogue.
+//   * masked keys (nonzero mask byte) cost the softmax nothing: GEMM 1 of a block that has some STARTS their accumulators
+//     at a value that loses every maximum and whose exponential is exactly 0; blocks whose keys are all masked are
+//     skipped.  The mask of a batch entry is classified once per workgroup, by wavefronts 0..3, in the prologue;
 //   * a second set of instantiations (FULLP) keeps P on all 255 steps of a byte - planned by the reference, README.md:15,186
 //     - by computing with P - 128 and starting the GEMM 2 accumulators at 128 times the column sums of the V tile.
 #include <hip/hip_runtime.h>
