@@ -110,11 +110,14 @@ int launch(hipStream_t stream, const FMHAParamI8& p, const FMHACrossAttnDescript
   args.floor2 = -1e6f * kLog2e;
   args.out_scale = output_scale(p);
   const dim3 grid((unsigned)args.total_wgs), block(fmha_i8_gfx950::kThreads);
-  // The accumulators of Q.K^T can be read as floats without a convert when they start at the bit pattern of kBase;
-  // the price is that the exponent offset (kBase*2^26 + S)*c2 is then rounded on a coarser float grid.  Take that path
-  // only while the offset stays below 2^12, i.e. while the rounding moves a whole row by less than 2^-13 in log2.
-  const bool bias = (fmha_i8_gfx950::kBase * fmha_i8_gfx950::kBaseScale + 4194304.f) * fabsf(args.c2) <
-                    fmha_i8_gfx950::kBiasOffsetLimit;
+  // The accumulators of Q.K^T can be read as floats without a convert when they start at the bit pattern of a float;
+  // the price is that the exponent offset (start value*2^26 + S)*c2 is then rounded on a coarser float grid.  Take that
+  // path only while the offset stays below 2^12, i.e. while the rounding moves a whole row by less than 2^-13 in log2.
+  // (The start value and the bound on |S| depend on the head size: see score_base_bits in the kernel source.)
+  const float offset_ulps = a.head_dim == 64
+                                ? fmha_i8_gfx950::score_base_ulps<64>() + fmha_i8_gfx950::score_range_ulps<64>()
+                                : fmha_i8_gfx950::score_base_ulps<128>() + fmha_i8_gfx950::score_range_ulps<128>();
+  const bool bias = offset_ulps * fabsf(args.c2) < fmha_i8_gfx950::kBiasOffsetLimit;
   // Folding the accumulator offset into the running O (see FASTACC in the kernel) costs a rounding of relative size
   // 2^-24 at magnitude kBase * sum(take) per key block; normalised by the row sum (>= sum(take)) and scaled to output
   // LSBs that is at most about 0.0034 * (v_amax/o_amax) * sqrt(key blocks).  Take it while that stays below 0.1 LSB.

@@ -63,6 +63,17 @@ constexpr float kMagic = 12582912.0f;    // 1.5 * 2^23: kMagic + y holds rne(y) 
 constexpr int kBaseBits = 0x3E22F983;
 constexpr float kBase = __builtin_bit_cast(float, kBaseBits);
 constexpr float kBaseScale = 67108864.0f;  // 2^26: float units per integer unit, inverted
+// The accumulators of GEMM 1 at head_dim 64 start lower in the same binade: 0x110000 = 1114112 ulps above 2^-3, more than
+// the 127*127*64 = 1032256 a dot product of 64 terms can reach.  The exponent offset of the biased path is rounded at the
+// magnitude (start value in ulps + S) * c2, and the lower start extends the range of score scales that path can serve by
+// a half (N(0,1) inputs at head_dim 64 fall inside it); GEMM 2 sums 128 keys whatever the head_dim and keeps kBaseBits.
+constexpr int kBaseBitsScores64 = 0x3E110000;
+template <int D>
+constexpr int score_base_bits() { return D == 64 ? kBaseBitsScores64 : kBaseBits; }
+template <int D>
+constexpr float score_base_ulps() { return (float)(score_base_bits<D>() - 0x3E000000) + 8388608.0f; }  // the start value / 2^-26
+template <int D>
+constexpr float score_range_ulps() { return D == 64 ? 1048576.0f : 4194304.0f; }  // bound on |S| used by the host
 constexpr float kBiasOffsetLimit = 4096.0f;  // see the launch code: bound on the exponent offset of the biased path
 constexpr float kLog2Pscale = -7.99995597f;  // log2(128 / 32767): exp2(x + kLog2Pscale) = 128 p / 32767
 constexpr float kLazyLog2 = 10.0f;       // the running O is rescaled only when a row maximum grows by more than this
@@ -136,8 +147,9 @@ __device__ __forceinline__ float half_sum(float x) {
   return __int_as_float(r[0]) + __int_as_float(r[1]);
 }
 
-// BIAS: the S accumulators start at kBaseBits and are read as floats (no int->float convert).  Exact only while
-// (kBase * 2^26 + |S|) * c2 stays small enough for the float grid; the host selects it from c2.
+// BIAS: the S accumulators start at the bit pattern of a float (kBaseBits; kBaseBitsScores64 at head_dim 64) and are read
+// as floats (no int->float convert).  Exact only while (start value * 2^26 + |S|) * c2 stays small enough for the float
+// grid; the host selects it from c2.
 // FASTACC: the running O absorbs the kBase offset of the GEMM 2 accumulators (one fma per element and key block
 // instead of subtract + fma) and the offset is taken out once, in the epilogue.  O then lives near kBase * sum(take)
 // and each merge rounds at that magnitude; the host enables it only where that rounding is far below one output LSB.
@@ -374,10 +386,12 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   float l_run;             // running row sum, in units of 1/128 (it sums 128*p)
   bool merged_any = false; // some key block has been merged into O, l and t
   const float c2 = BIAS ? args.c2 * kBaseScale : args.c2;  // exponent per unit of sf() below
-  const float bias_c2 = BIAS ? kBase * c2 : 0.f;
+  constexpr int kScoreBaseBits = score_base_bits<D>();  // start value of the GEMM 1 accumulators on the BIAS variant
+  const float bias_c2 = BIAS ? __builtin_bit_cast(float, kScoreBaseBits) * c2 : 0.f;
   float magic;
   int flip_top;
-  v16i base_c;
+  v16i base_c;             // start value of the GEMM 2 accumulators (and of GEMM 1 at head_dim 128), in sixteen registers
+  v16i base_s;             // start value of the GEMM 1 accumulators
   v4i qreg[kDSteps];       // Q: B operand of GEMM 1, loaded once
   int kb_end = 0;          // one past the last key block that holds any unmasked key (trailing padding is never computed on)
   int kb_plain = 0;        // the first block with any masked key: blocks [0, kb_plain) have none
@@ -398,6 +412,14 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     base_c = v16i{kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits,
                   kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits, kBaseBits};
     asm volatile("" : "+v"(base_c));  // held in registers: as a known constant it is rebuilt by eight moves per key block
+    if (kScoreBaseBits == kBaseBits) {
+      base_s = base_c;
+    } else {
+      base_s = v16i{kScoreBaseBits, kScoreBaseBits, kScoreBaseBits, kScoreBaseBits, kScoreBaseBits, kScoreBaseBits,
+                    kScoreBaseBits, kScoreBaseBits, kScoreBaseBits, kScoreBaseBits, kScoreBaseBits, kScoreBaseBits,
+                    kScoreBaseBits, kScoreBaseBits, kScoreBaseBits, kScoreBaseBits};
+      if (BIAS) asm volatile("" : "+v"(base_s));
+    }
   };
 
   // ---- the prologue ------------------------------------------------------------------------------------------------
@@ -618,7 +640,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         const unsigned lo = (unsigned)(((int)(mw[t] << (31 - key))) >> 31), hi = (unsigned)(((int)(mw[t] << (27 - key))) >> 31);
         const unsigned long long lanes = ((unsigned long long)hi << 32) | lo;
         int e;
-        if (BIAS) asm volatile("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(e) : "v"(base_c[0]), "v"(gone), "s"(lanes));
+        if (BIAS) asm volatile("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(e) : "v"(base_s[0]), "v"(gone), "s"(lanes));
         else asm volatile("v_cndmask_b32_e64 %0, 0, %1, %2" : "=v"(e) : "v"(gone), "s"(lanes));
         acc[t][r] = e;
       }
@@ -663,7 +685,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       for (int kk = 0; kk < kDSteps; ++kk) {
         align8();
         acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ka[t & 1][kk], qreg[kk],
-                                                       kk == 0 ? (BIAS ? base_c : zero_c) : acc[t], 0, 0, 0);
+                                                       kk == 0 ? (BIAS ? base_s : zero_c) : acc[t], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         if (t >= 1) {
 #pragma unroll
@@ -674,7 +696,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       }
     }
   };
-  // (sf(t,r) below: the score as a float; with BIAS that is kBase + S * 2^-26, and the exponent offset removes kBase.)
+  // (sf(t,r) below: the score as a float; with BIAS that is the start value + S * 2^-26, and the exponent offset removes the start value.)
   // block softmax (inc/fmha_i8.cuh:174-253)
   // split = false: the whole block softmax, P packed, software-pipelined (the general loop).  split = true (the
   // steady-state loop): everything but the P packing, in three dense runs - 64 scale fmas, 64 exponentials, 64 + 4 adds -
@@ -698,7 +720,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       for (int j = 0; j < 4; ++j) tile_max_piece(acc[kKeyTiles - 1], mx, false, j);
       int ti = half_max(max(mx[0], mx[1]));
       // a masked key enters the maximum as the integer -1000000 (inc/fmha_i8.cuh:191-193)
-      if (cls != 0) ti = max(ti, (BIAS ? kBaseBits : 0) - 1000000);
+      if (cls != 0) ti = max(ti, (BIAS ? kScoreBaseBits : 0) - 1000000);
       const float top = BIAS ? __int_as_float(ti) : (float)ti;
       // off = top*c2 rounded; p' = exp2(s*c2 - off) = p * 2^(resid) with one row-wide resid below 1 ulp of off, and the
       // block maximum that is consistent with p' is off itself (minus the constant kBase*c2 when BIAS).

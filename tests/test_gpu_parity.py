@@ -261,6 +261,26 @@ def test_every_kernel_variant(pkg, orc, dev, S, d, qk_scale, vo_ratio):
     check(gpu_run(pkg, dev, c, **kw), want, "variant S=%d d=%d qk=%g vo=%g" % (S, d, qk_scale, vo_ratio))
 
 
+@pytest.mark.parametrize("d", [64, 128])
+def test_extreme_scores_stay_inside_the_float_window(pkg, orc, dev, d):
+    """On the variant that reads the GEMM 1 accumulators as floats, the accumulators start inside a float binade and
+    the largest possible |S| = 127*127*d must not leave it (at head_dim 64 the start value sits closer to the lower
+    edge than at 128).  Rows of +-127 reach both extremes; a tiny score scale selects that variant and keeps the
+    softmax non-trivial (x = S*c differs by a few units across keys)."""
+    S = 256
+    rng = np.random.default_rng(d)
+    q = np.full((1, 2, S, d), 127, np.int8)
+    q[0, 1, ::2] = -127
+    k = np.where(rng.random((1, 2, S, 1)) < 0.5, 127, -127).astype(np.int8) * np.ones((1, 1, 1, d), np.int8)
+    k[0, :, 5, :] = rng.integers(-127, 128, (2, d))  # one ordinary key per head
+    v = rng.integers(-127, 128, (1, 2, S, d)).astype(np.int8)
+    mask = np.zeros((1, S), np.int8)
+    mask[0, 200:230] = 1
+    c = dict(q=q, k=k, v=v, mask=mask, q_amax=0.02, k_amax=0.02, v_amax=1.0, o_amax=1.0)
+    want = cpu_run(orc, c)
+    check(gpu_run(pkg, dev, c), want, "extreme scores d=%d" % d)
+
+
 # Key blocks come in three kinds - no masked key (P), some (M), all (F) - and the kernel serves them with three loops
 # (a steady-state loop for runs of P, a second one from the first M on, a general loop for F blocks and the last
 # block); masked keys of an M block are handled where GEMM 1 starts its accumulators.  Every transition between the
