@@ -268,10 +268,12 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
                  :: "s"(dst), "v"(src), "s"(gbase) : "memory");
   };
   bool prologue_done = false;  // (the test build without tile loads still fetches the tiles of the prologue)
-  auto issue_region = [&](const int8_t* gbase, int kb, int which, int goff, int it) __attribute__((always_inline)) {  // which: 0 = K, 1 = V
+  // (steady: called from a steady-state loop, which a sequence of less than one key block never enters - said at compile
+  // time, so that those loops carry no branch for it)
+  auto issue_region = [&](const int8_t* gbase, int kb, int which, int goff, int it, bool steady = false) __attribute__((always_inline)) {  // which: 0 = K, 1 = V
     if (test_build::kNoTileLoads && prologue_done) return;
     const int region = (it * kWaves + wave) % kRegions;
-    if (RAGGED && short_seq) {
+    if (RAGGED && !steady && short_seq) {
       issue_short_region(gbase, which, goff, region);
       return;
     }
@@ -331,8 +333,12 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // an address that is 4 mod 8 (one instruction per fetch of an aligned pair of dwords); the compiler aligns nothing
   // inside a function.  The d = 64 kernel is sensitive to where the MFMAs of GEMM 1 and the row-maximum instructions
   // behind them fall (+12 % when they straddle), so it pins those, the scale fmas and the P packing to aligned
-  // addresses; the d = 128 kernel measures the same either way (+-0.3 %) and is left alone.
-  auto align8 = [&]() { if (D == 64) asm volatile(".p2align 3" ::: "memory"); };
+  // addresses; the d = 128 kernel measures the same either way (+-0.3 %) in its loop without masked keys and is left
+  // alone there (pinning everything costs it 0.4 %).  Its loop for blocks WITH masked keys is sensitive (up to 9 % between
+  // two placements, B1 H4 S8192 with a scattered mask), so that loop pins the same groups, and GEMM 1 with start values
+  // pins each tile's run of v_cndmask and its MFMAs at either head size: 1.5 to 3 % faster and 3 % left between
+  // placements.
+  auto align8 = [&](bool also_at_128 = false) { if (D == 64 || also_at_128) asm volatile(".p2align 3" ::: "memory"); };
   // The steady-state loops start at a fixed distance from a 64-byte boundary, so that what is measured for them does
   // not change with the code in front of them: at d = 64 the loop of wavefronts 0..3 runs 12 % slower when it starts
   // 4 bytes further on or back (B16 H16 S2048: 226 against 254 us; every even distance measures the same, every odd
@@ -342,8 +348,9 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // (the test builds loop_pad_a0 and loop_pad_a1, -DFMHA_LOOP_PAD_A=0 against 1) whenever the code between the boundary
   // and the loop changes; tests/test_gpu_variant_builds.py holds the shipped library to the faster of the two.
   auto align_loop = [&]() { asm volatile(".p2align 6" ::: "memory"); };
-  // s_nops between the boundary and the loop of wavefronts 0..3 (see above)
-  constexpr int kLoopPadA = test_build::kLoopPadA >= 0 ? test_build::kLoopPadA : 0;
+  // s_nops between the boundary and the loop of wavefronts 0..3 (see above): the 255-step variant has other code
+  // between the two and wants the odd distance (d = 64, B16 H16 S2048: 243 against 257 us)
+  constexpr int kLoopPadA = test_build::kLoopPadA >= 0 ? test_build::kLoopPadA : (FULLP && D == 64) ? 1 : 0;
   // (test build with time stamps: every wavefront records the shader clock at each barrier arrival and departure, in the
   // lanes of one register; lanes 62 and 63 take the constant-rate 100 MHz counter when the wavefront starts and ends,
   // which with the first and the last stamp gives the shader clock the kernel actually ran at)
@@ -370,8 +377,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   auto barrier = [&]() { stamp(); asm volatile("s_barrier" ::: "memory"); stamp(); };
 
   // One workgroup barrier per key block, or (a test build) two: see the schedule below.
-  // (FULLP at d = 64 keeps two: with one it measures 10 % slower, at d = 128 4 to 7 % faster.)
-  constexpr bool kOneBarrier = !test_build::kTwoBarriers && !(FULLP && D == 64);
+  constexpr bool kOneBarrier = !test_build::kTwoBarriers;
   constexpr int kVAhead = (FULLP && kOneBarrier) ? 3 : 2;
 
   const int row0 = qb * kBlockQ + wave * 32;  // first query row of this wavefront
@@ -465,8 +471,16 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       if (!RAGGED || S >= kKeysPerLane)  // (a shorter mask row has no 16 bytes that lie inside it)
         asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(mask_bytes) : "v"(j), "s"(mg) : "memory");
     }
+    // RAGGED: the last sixteen mask bytes of the row, for the one lane whose sixteen keys straddle its end
+    v4i tail_bytes = {0, 0, 0, 0};
+    if (RAGGED && S >= kKeysPerLane) {
+      int j = S - kKeysPerLane;
+      if (!fmha_in_bounds(j >= 0 && j + kKeysPerLane <= S)) j = 0;
+      asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(tail_bytes) : "v"(j), "s"(mg) : "memory");
+    }
     load_q_rows();
     asm volatile("s_waitcnt vmcnt(%1)" : "+v"(mask_bytes) : "n"(kDSteps) : "memory");
+    asm volatile("" : "+v"(tail_bytes));
     constexpr int kLanesPerBlock = BK / kKeysPerLane;
     constexpr int kBlocksPerWave = 64 / kLanesPerBlock;
     constexpr unsigned long long kGroupBits = kLanesPerBlock == 8 ? 0x0101010101010101ull : 0x1111111111111111ull;
@@ -488,7 +502,14 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         bits = nonzero_bytes((unsigned)w[0]) | (nonzero_bytes((unsigned)w[1]) << 4) | (nonzero_bytes((unsigned)w[2]) << 8) |
                (nonzero_bytes((unsigned)w[3]) << 12);
       } else if (RAGGED && j < S) {  // the one lane that straddles the end
-        for (int b = 0; b < S - j; ++b) bits = (mg[fmha_in_bounds(j + b < S) ? j + b : 0] != 0) ? bits : (bits & ~(1u << b));
+        if (S >= kKeysPerLane) {
+          // its S - j keys are the last S - j of the row's last sixteen
+          const unsigned last16 = nonzero_bytes((unsigned)tail_bytes[0]) | (nonzero_bytes((unsigned)tail_bytes[1]) << 4) |
+                                  (nonzero_bytes((unsigned)tail_bytes[2]) << 8) | (nonzero_bytes((unsigned)tail_bytes[3]) << 12);
+          bits = ((last16 >> (kKeysPerLane - (S - j))) | (0xffffu << (S - j))) & 0xffffu;
+        } else {
+          for (int b = 0; b < S - j; ++b) bits = (mg[fmha_in_bounds(j + b < S) ? j + b : 0] != 0) ? bits : (bits & ~(1u << b));
+        }
       }
       // two lanes hold the 32 mask bits of one word
       const unsigned word = bits | ((unsigned)__shfl_xor((int)bits, 1) << 16);
@@ -653,12 +674,13 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       for (int t = 0; t < kKeyTiles; ++t) {
 #pragma unroll
         for (int kk = 0; kk < kDSteps; ++kk) ka[0][kk] = read_k(k_read_off[kk] + 32 * t * D);
+        align8(true);
         start_piece(t, 0, 16);
         asm volatile("s_nop 1" ::: "memory");  // (the compiler does not know that the statements above wrote registers an MFMA reads)
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int kk = 0; kk < kDSteps; ++kk) {
-          align8();
+          align8(true);
           acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ka[0][kk], qreg[kk], acc[t], 0, 0, 0);
           __builtin_amdgcn_sched_barrier(0);
           if (t >= 1) {
@@ -701,7 +723,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // split = false: the whole block softmax, P packed, software-pipelined (the general loop).  split = true (the
   // steady-state loop): everything but the P packing, in three dense runs - 64 scale fmas, 64 exponentials, 64 + 4 adds -
   // and the exponentials are left in acc (as float bits) for phase_pack, which runs at the head of the MFMA phase.
-  auto phase_softmax = [&](int kb, int cls, v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles], int (&mx)[2], bool split = false) __attribute__((always_inline)) {
+  auto phase_softmax = [&](int kb, int cls, v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles], int (&mx)[2], bool split = false, bool aligned = false) __attribute__((always_inline)) {
     if constexpr (test_build::kNoSoftmax) {
       if (!split) {
 #pragma unroll
@@ -744,7 +766,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         // class: measured against the pipelined form with the packing left to the compiler's placement, -6 % at d = 64
         // (where it also makes one barrier per key block the faster choice) and level at d = 128.
         float xs[kQuads][4];
-        align8();
+        align8(aligned);
 #pragma unroll
         for (int qd = 0; qd < kQuads; ++qd)
 #pragma unroll
@@ -855,13 +877,13 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
     }
   };
   // P packing of the exponentials that phase_softmax(split) left in acc: P^T as the B operand of GEMM 2.
-  auto phase_pack = [&](v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles]) __attribute__((always_inline)) {
+  auto phase_pack = [&](v16i (&acc)[kKeyTiles], v4i (&pk)[kKeyTiles], bool aligned = false) __attribute__((always_inline)) {
     if constexpr (test_build::kNoSoftmax) {
 #pragma unroll
       for (int t = 0; t < kKeyTiles; ++t) test_build::undefined(pk[t]);
       return;
     }
-    align8();
+    align8(aligned);
 #pragma unroll
     for (int qd = 0; qd < 4 * kKeyTiles; ++qd) {
       float e[4];
@@ -896,7 +918,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // registers, which needs the loads of a key block in one place.
   constexpr bool kLoadsInMfmaPhase = !test_build::kStagedLoads || D == 64;
   static_assert(!kLoadsInMfmaPhase || 2 * kRegionsPerWave <= kDSteps, "one tile load per output tile of GEMM 2");
-  auto phase_gemm2_merge = [&](int kb, const v4i (&pk)[kKeyTiles], int k_next, int v_next) __attribute__((always_inline)) {
+  auto phase_gemm2_merge = [&](int kb, const v4i (&pk)[kKeyTiles], int k_next, int v_next, bool steady = false) __attribute__((always_inline)) {
     if constexpr (test_build::kNoMfma) {
       if (kLoadsInMfmaPhase) {
         issue_k(k_next);
@@ -988,8 +1010,8 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
         }
       }
       if (kLoadsInMfmaPhase) {
-        if (u < kRegionsPerWave) issue_region(kg, k_next, 0, ld_goff_k, u);
-        else if (u < 2 * kRegionsPerWave) issue_region(vg, v_next, 1, ld_goff_v, u - kRegionsPerWave);
+        if (u < kRegionsPerWave) issue_region(kg, k_next, 0, ld_goff_k, u, steady);
+        else if (u < 2 * kRegionsPerWave) issue_region(vg, v_next, 1, ld_goff_v, u - kRegionsPerWave, steady);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -1124,7 +1146,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       v4i pk[kKeyTiles];
       wait_v_for_colsum_a();
       barrier_odd();
-      phase_softmax(i, cls, acc, pk, mx, kSplitSoftmax);
+      phase_softmax(i, cls, acc, pk, mx, kSplitSoftmax, next_masked);
       if (kSplitSoftmax) pin_scores(acc);
       issue_after_softmax_a(i);
       staged_writes_done();
@@ -1135,9 +1157,9 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       raise_priority();
       if (kSplitSoftmax) {
         pin_scores(acc);
-        phase_pack(acc, pk);
+        phase_pack(acc, pk, next_masked);
       }
-      phase_gemm2_merge(i, pk, min(i + 3, last), min(i + kVAhead, last));
+      phase_gemm2_merge(i, pk, min(i + 3, last), min(i + kVAhead, last), true);
       if (next_masked) phase_gemm1(i + 1, acc, mx, true);
       else phase_gemm1(i + 1, acc, mx, false);
       drop_priority();
@@ -1196,7 +1218,7 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       v4i pk[kKeyTiles];
       wait_tiles(false);
       barrier();
-      phase_softmax(i, cls, acc, pk, mx, kSplitSoftmax);
+      phase_softmax(i, cls, acc, pk, mx, kSplitSoftmax, next_masked);
       if (kSplitSoftmax) pin_scores(acc);
       if (kStaged) staged_step(i);
       else issue_after_softmax(i);
@@ -1205,9 +1227,9 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
       raise_priority();
       if (kSplitSoftmax) {
         pin_scores(acc);
-        phase_pack(acc, pk);
+        phase_pack(acc, pk, next_masked);
       }
-      phase_gemm2_merge(i, pk, min(i + 3, last), min(i + kVAhead, last));
+      phase_gemm2_merge(i, pk, min(i + 3, last), min(i + kVAhead, last), true);
       if (FULLP) phase_colsum(i + 1);
       if (next_masked) phase_gemm1(i + 1, acc, mx, true);
       else phase_gemm1(i + 1, acc, mx, false);
