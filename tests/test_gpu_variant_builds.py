@@ -86,46 +86,54 @@ def test_two_barrier_build_writes_the_shipped_bytes_on_every_kind_of_instantiati
         assert np.array_equal(got, want), ((B, H, S, d, dist, pad, full), int((got != want).sum()))
 
 
-def _time_us(lib, pkg, dev, c, calls):
+def _time_us(lib, pkg, dev, c, calls, full_range_p=False):
     import time
 
     import torch
     lib.FMHAInferI8Status.argtypes = [C.c_void_p, pkg.FMHAParamI8, pkg.AttnDataDescriptor] + [C.c_void_p] * 5 + [C.c_bool]
     lib.FMHAInferI8Status.restype = C.c_int
+    lib.FMHAInferI8CrossFullRangeP.argtypes = [C.c_void_p, pkg.FMHAParamI8, pkg.FMHACrossAttnDescriptor] + [C.c_void_p] * 5
+    lib.FMHAInferI8CrossFullRangeP.restype = C.c_int
     B, H, S, d = c["q"].shape
     q, k, v, m = (torch.from_numpy(np.ascontiguousarray(c[n])).to(dev) for n in ("q", "k", "v", "mask"))
     o = torch.empty_like(q)
     stream = torch.cuda.current_stream(dev)
-    args = (stream.cuda_stream, pkg.FMHAParamI8(c["q_amax"], c["k_amax"], c["v_amax"], c["o_amax"], 1.0),
-            pkg.AttnDataDescriptor(B, S, H, d), q.data_ptr(), k.data_ptr(), v.data_ptr(), m.data_ptr(), o.data_ptr(), True)
+    scales = pkg.FMHAParamI8(c["q_amax"], c["k_amax"], c["v_amax"], c["o_amax"], 1.0)
+    pointers = (q.data_ptr(), k.data_ptr(), v.data_ptr(), m.data_ptr(), o.data_ptr())
+    if full_range_p:
+        fn, args = lib.FMHAInferI8CrossFullRangeP, (stream.cuda_stream, scales, pkg.FMHACrossAttnDescriptor(B, S, S, H, d)) + pointers
+    else:
+        fn, args = lib.FMHAInferI8Status, (stream.cuda_stream, scales, pkg.AttnDataDescriptor(B, S, H, d)) + pointers + (True,)
     t0 = time.perf_counter()
     while time.perf_counter() - t0 < 0.08:  # the shader clock settles
         for _ in range(50):
-            assert lib.FMHAInferI8Status(*args) == 0
+            assert fn(*args) == 0
         torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     best = 1e30
     for _ in range(3):
         e0.record(stream)
         for _ in range(calls):
-            lib.FMHAInferI8Status(*args)
+            fn(*args)
         e1.record(stream)
         torch.cuda.synchronize()
         best = min(best, e0.elapsed_time(e1) * 1e3 / calls)
     return best
 
 
-def test_the_steady_state_loop_sits_where_it_runs_fast(pkg, dev):
-    """At d = 64 the loop of wavefronts 0..3 runs 12 % slower when it starts 4 bytes off (see align_loop in the kernel
-    source), and which of the two placements is the fast one changes with the code in front of the loop.  The shipped
-    library must be as fast as the faster of the two test builds that pin the placement either way."""
+@pytest.mark.parametrize("full_range_p", [False, True], ids=["P_128_steps", "P_255_steps"])
+def test_the_steady_state_loop_sits_where_it_runs_fast(pkg, dev, full_range_p):
+    """At d = 64 the loop of wavefronts 0..3 runs 6 to 12 % slower when it starts 4 bytes off (see align_loop in the
+    kernel source), and which of the two placements is the fast one changes with the code in front of the loop - it is
+    not the same for the 128-step and the 255-step kernel.  The shipped library must be as fast as the faster of the two
+    test builds that pin the placement either way."""
     c = fc.make_inputs(16, 16, 2048, 64, dist="student_t", sigma=0.5, pad="none", seed=7)
     shipped = pkg.load_library()
-    times = {"shipped": _time_us(shipped, pkg, dev, c, 100)}
+    times = {"shipped": _time_us(shipped, pkg, dev, c, 100, full_range_p)}
     for name in ("loop_pad_a0", "loop_pad_a1"):
         path = os.path.join(HERE, "bin", "libfmha_i8_%s.so" % name)
         assert os.path.exists(path), "%s is missing: build it with `make -C tests all`" % path
-        times[name] = _time_us(C.CDLL(path), pkg, dev, c, 100)
-    times["shipped"] = min(times["shipped"], _time_us(shipped, pkg, dev, c, 100))  # before and after: board power drifts
+        times[name] = _time_us(C.CDLL(path), pkg, dev, c, 100, full_range_p)
+    times["shipped"] = min(times["shipped"], _time_us(shipped, pkg, dev, c, 100, full_range_p))  # before and after: board power drifts
     print(times, flush=True)
-    assert times["shipped"] <= 1.04 * min(times["loop_pad_a0"], times["loop_pad_a1"]), times
+    assert times["shipped"] <= 1.03 * min(times["loop_pad_a0"], times["loop_pad_a1"]), times
