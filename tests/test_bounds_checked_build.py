@@ -48,7 +48,8 @@ def test_checked_build_counts_nothing_on_any_shape(pkg, orc, checked, dev):
     assert checked.FMHAInferI8DebugOutOfBounds() == 0  # (also clears the counter)
     rng = np.random.default_rng(77)
     shapes = [(3, 3, 319, 3, 64), (1, 1, 1, 1, 128), (2, 2, 70, 70, 128), (2, 1, 300, 129, 64), (1, 2, 64, 64, 64),
-              (1, 2, 1024, 1024, 128), (2, 2, 2048, 2048, 64), (1, 1, 100, 4095, 128), (1, 1, 4097, 65, 64)]
+              (1, 2, 1024, 1024, 128), (2, 2, 2048, 2048, 64), (1, 1, 100, 4095, 128), (1, 1, 4097, 65, 64),
+              (2, 1, 40, 15, 64), (2, 1, 40, 16, 128), (2, 1, 40, 17, 64), (2, 1, 40, 31, 128), (1, 1, 40, 4100, 64)]
     for _ in range(40):
         S = int(rng.choice([rng.integers(1, 130), rng.integers(1, 700), rng.integers(500, 2600), 64 * rng.integers(1, 40)]))
         Sq = S if rng.random() < 0.4 else int(rng.choice([rng.integers(1, 70), rng.integers(1, 600), rng.integers(200, 1500)]))

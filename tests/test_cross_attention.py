@@ -187,6 +187,27 @@ def test_any_key_count(pkg, orc, dev, S, d):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("S", [15, 16, 17, 31, 33, 4100, 4111])
+def test_mask_bytes_of_the_lane_that_straddles_the_end_of_the_row(pkg, orc, dev, S, d):
+    """The kernel classifies the mask sixteen bytes per lane; the lane whose sixteen keys straddle the end of the row
+    takes its bytes from the row's last sixteen (one load that ends where the row ends), rows shorter than sixteen
+    bytes are read byte by byte, and rows of more than 4096 keys are classified in several passes.  A scattered mask,
+    so that every one of those bytes shows in the output."""
+    B, H, Sq = 2, 2, 77
+    Sp = (S + 63) // 64 * 64
+    c = fc.make_inputs(B, H, Sp, d, pad="scatter", seed=66)
+    c["mask"][:, 0] = 0
+    c["mask"][0, S - 1] = 0  # the last key of the row: attended to in one batch entry, masked out in the other
+    c["mask"][1, S - 1] = 1
+    cut = dict(c, k=c["k"][:, :, :S], v=c["v"][:, :, :S], mask=c["mask"][:, :S])
+    cut = {n: (np.ascontiguousarray(a) if isinstance(a, np.ndarray) else a) for n, a in cut.items()}
+    q = fc.make_inputs(B, H, Sq, d, seed=67)["q"]
+    _gate(_gpu(pkg, dev, q, cut, canary=True), orc.fmha_i8_blockwise_cross(q, cut["k"], cut["v"], cut["mask"], *_scales(c)),
+          "S=%d d=%d" % (S, d))
+
+
+@pytest.mark.gpu
 def test_any_key_count_at_the_end_of_an_allocation(pkg, orc, dev):
     """K, V and the mask end exactly where their device allocations end: a tile load or a mask read that ran past the
     last key would leave the buffers (the last head of the last batch entry is the one that matters)."""
