@@ -103,6 +103,8 @@ def main():
                     wait[w // 4].append(dx[1::2][3:-3])
                     work[w // 4].append(dx[2::2][3:-3])
         for grp, name in ((0, "wavefronts 0-3"), (1, "wavefronts 4-7")):
+            if not work[grp]:  # too few key blocks for a steady state
+                continue
             wk, wt = np.concatenate(work[grp]), np.concatenate(wait[grp])
             out["ticks_" + name.replace(" ", "_")] = {
                 "work_between_barriers_mean": round(float(wk.mean()), 1), "wait_at_barrier_mean": round(float(wt.mean()), 1),
