@@ -1127,7 +1127,17 @@ __global__ __launch_bounds__(kThreads, 2) void fmha_i8_fwd_kernel(const KernelAr
   // The wavefront in its MFMA phase gets the issue slots it asks for: an MFMA, an operand read or a merge instruction
   // that waits behind the other wavefront's softmax stream leaves the MFMA pipe idle, the reverse costs nothing.
   auto raise_priority = [&]() { asm volatile("s_setprio 3" ::: "memory"); };
-  auto drop_priority = [&]() { asm volatile("s_setprio 0" ::: "memory"); };
+  // Outside the MFMA phase wavefronts 0..3 run at priority 0.  Wavefronts 4..7 keep priority 1 there in the d = 64 kernel
+  // that reads its scores without a conversion: when both wavefronts of a SIMD are in the softmax the older one (0..3)
+  // otherwise wins every issue slot, and the workgroup starts with 4..7 behind.  Measured: B8 H12 S512 9.87 -> 9.57 us,
+  // B32 H12 S256 13.15 -> 12.38, B64 H12 S384 45.7 -> 43.7, S2048 level; the converting d = 64 kernel loses 2 to 6 % from
+  // 1024 keys on and the d = 128 kernels move by less than 1 % either way, so they stay at 0.  (Levels 1, 2 and 3
+  // measure the same; the instruction has one length, so no code moves.)
+  constexpr int kSoftmaxPriority47 = (D == 64 && BIAS) ? 1 : 0;
+  auto drop_priority = [&]() {
+    if (kSoftmaxPriority47 != 0 && wave >= kClassWaves) asm volatile("s_setprio %0" :: "n"(kSoftmaxPriority47) : "memory");
+    else asm volatile("s_setprio 0" ::: "memory");
+  };
   if (wave < kClassWaves) {
     prologue_waves_0_to_3();
     first_barrier();
